@@ -1,0 +1,122 @@
+/*
+ * pbs_hip.h -- C ABI of libpbs_hip.so, the MI355X (gfx950) block-sparse matmul engine.
+ *
+ * Plain C: raw device pointers, sizes and a hipStream_t passed as void*.  No torch
+ * types.  All pointers are caller-owned device memory; the library keeps nothing
+ * after a call returns and holds no mutable global device state, so calls on
+ * different streams or from different host threads do not interfere.
+ *
+ * Every entry point returns an int: 0 on success, a positive hipError_t when the HIP
+ * runtime reported an error, a negative PBS_ERR_* when an argument was rejected
+ * before anything was launched.  pbs_error_string() turns either into text.
+ *
+ * Data conventions (those of the reference's BlockSparseMatrix, block_sparse.py):
+ *   - the weight W is [out_features, in_features], tiled in 32x32 blocks; X = out/32
+ *     block rows, Y = in/32 block columns, nnz nonzero blocks;
+ *   - packed data is [nnz*32, 32] row-major; data block b holds its W block
+ *     transposed: data[32b + j][i] = W[32r + i][32c + j]      (block_sparse.py:326-331)
+ *   - row_start_ends_a [X+1], cols_a [nnz][2] = (block col, data block)   CSR
+ *   - col_start_ends_b [Y+1], rows_b [nnz][2] = (block row, data block)   CSC
+ *   - blocks [nnz][2] = (block col, block row) of data block b         (:138-141)
+ *   - dense operands are row-major and contiguous; dense results are row-major.
+ */
+#ifndef PBS_HIP_H
+#define PBS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PBS_ABI_VERSION 1
+#define PBS_BLOCK 32
+
+/* element type of dense operands, packed data and results (accumulation is fp32) */
+#define PBS_DTYPE_F32 0
+#define PBS_DTYPE_BF16 1
+
+#define PBS_OK 0
+#define PBS_ERR_NULL_POINTER (-1)
+#define PBS_ERR_BAD_SHAPE (-2)     /* negative size or a feature dim not a multiple of 32 */
+#define PBS_ERR_BAD_DTYPE (-3)
+#define PBS_ERR_MISALIGNED (-4)    /* a dense/data pointer is not 16-byte aligned */
+#define PBS_ERR_WORKSPACE (-5)     /* workspace missing or smaller than pbs_*_workspace_bytes */
+#define PBS_ERR_TOO_LARGE (-6)     /* a size exceeds what the kernels index with */
+
+int pbs_abi_version(void);
+const char* pbs_error_string(int code);
+
+/*
+ * Index arrays of a block mask, built on the device, bit-exact with the reference's
+ * BlockSparseMatrixBase.build_indices (block_sparse.py:125-153, helper :85-123).
+ *
+ *   mask       [X*Y] bytes, row-major, nonzero = block present
+ *   block_ptr  NULL, or [nnz] int64: data-block id of the i-th nonzero in row-major
+ *              order (the "recycled blocks" path used by block_replace, :210-219)
+ *   nnz        the number of blocks the caller allocated outputs for
+ *   status     [2] int32 device words: status[0] = number of nonzeros counted in mask,
+ *              status[1] = 0 if ok, 1 if the count differs from nnz (nothing else is
+ *              written then), 2 if a block_ptr entry is outside [0, nnz)
+ */
+int pbs_build_indices(const uint8_t* mask, const int64_t* block_ptr, int X, int Y, int nnz,
+                      int32_t* cols_a, int32_t* row_start_ends_a,
+                      int32_t* rows_b, int32_t* col_start_ends_b,
+                      int32_t* blocks, int32_t* status, void* stream);
+
+/*
+ * dense x block-sparse -> dense.  Replaces blocksparse_matmul_cutlass
+ * (native/block_sparse_native.cpp:6-16, launcher native/block_sparse_cutlass_kernel.cu:113-150)
+ * as called by BlockSparseMatrixBase.reverse_matmul_ (block_sparse.py:496-578).
+ *
+ *   transpose = 1 : out[tokens, n] = a[tokens, k] . W^T   n = out_features, k = in_features,
+ *                   ptr = row_start_ends_a, indices = cols_a          (forward, :518-521)
+ *   transpose = 0 : out[tokens, n] = a[tokens, k] . W     n = in_features,  k = out_features,
+ *                   ptr = col_start_ends_b, indices = rows_b          (input gradient, :522-525)
+ *
+ * Differences from the reference entry point, all on purpose: `data` is always the
+ * packed data as stored (no per-call transposed copy of the weights, :541-544); `out`
+ * is row-major [tokens, n] and need not be zeroed (the reference wants a zeroed
+ * [n, tokens] buffer, :516); `bias` is NULL or [n] and is added in the epilogue
+ * (the reference adds it in a separate pass, block_sparse_linear.py:231-232);
+ * any tokens >= 0 is handled; work is launched on `stream`, not on stream 0.
+ */
+int pbs_blocksparse_matmul(const void* dense_a, const void* data,
+                           const int32_t* ptr, const int32_t* indices,
+                           const void* bias, void* dense_out,
+                           int64_t tokens, int n, int k, int nnz,
+                           int transpose, int dtype, void* stream);
+
+/*
+ * dense^T x dense -> block-sparse (only the nonzero blocks are computed), packed like
+ * `data`:  out[32b + j][i] = sum_t dense_a[t][32r + i] * dense_b[t][32c + j].
+ * Replaces blocksparse_matmul_back_cutlass (native/block_sparse_native.cpp:18-29,
+ * launcher native/block_sparse_cutlass_kernel_back.cu:118-160) as called by
+ * matmul_with_output_sparse_support_ (block_sparse.py:606-655); result layout as in
+ * cutlass/gemm/block_task_back.h:537-538.
+ *
+ *   dense_a [tokens, out_features] (grad_output), dense_b [tokens, in_features] (input),
+ *   both row-major contiguous.  The pattern is given by the CSR pair
+ *   (row_start_ends_a, cols_a) instead of the reference's `blocks` list so that a
+ *   workgroup can find the blocks of its tile of W without scanning all of them.
+ *   Every token is accumulated (the reference drops tokens % 32 when tokens > 32).
+ *   `out` need not be zeroed.
+ *
+ * When the tile grid alone cannot fill the GPU the token range is split over
+ * workgroups and the fp32 partial blocks are summed in a fixed order by a second
+ * kernel; that needs `workspace` of pbs_blocksparse_matmul_back_workspace_bytes()
+ * bytes (16-byte aligned device memory; may be NULL when that returns 0).
+ */
+size_t pbs_blocksparse_matmul_back_workspace_bytes(int64_t tokens, int out_features, int in_features,
+                                                   int nnz, int dtype);
+int pbs_blocksparse_matmul_back(const void* dense_a, const void* dense_b,
+                                const int32_t* row_start_ends_a, const int32_t* cols_a,
+                                void* data_out,
+                                int64_t tokens, int out_features, int in_features, int nnz,
+                                int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PBS_HIP_H */

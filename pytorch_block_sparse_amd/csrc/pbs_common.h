@@ -1,0 +1,102 @@
+// Shared device helpers for the gfx950 block-sparse kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace pbs {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+struct bf16_t {
+    uint16_t bits;
+};
+
+// Per element type: bytes, and how one 32x32x32 block product is issued on the matrix cores.
+//
+// A "fragment" is what one lane holds of a 32(rows) x 32(k) operand tile: lane l serves row
+// (l & 31) and the 16 consecutive k values 16*(l >> 5) .. +15, kept as NQ 16-byte registers
+// quads.  Both operands of a product use the same assignment of k to (lane half, register),
+// so any operand whose k runs contiguously in memory is loaded with plain 16-byte reads.
+template <typename T>
+struct Elem;
+
+template <>
+struct Elem<float> {
+    static constexpr int ESZ = 4;
+    static constexpr int NQ = 4;  // 16 floats per lane
+    // v_mfma_f32_32x32x2_f32: lane half h supplies k = h of each 2-wide step; here step
+    // (q, e) contracts the k pair {4q+e, 16+4q+e}.
+    static __device__ __forceinline__ void mma(f32x16& acc, const uint4* a, const uint4* b) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[q].x), __uint_as_float(b[q].x), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[q].y), __uint_as_float(b[q].y), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[q].z), __uint_as_float(b[q].z), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[q].w), __uint_as_float(b[q].w), acc, 0, 0, 0);
+        }
+    }
+    static __device__ __forceinline__ float from_f32(float v) { return v; }
+    static __device__ __forceinline__ float to_f32(float v) { return v; }
+};
+
+template <>
+struct Elem<bf16_t> {
+    static constexpr int ESZ = 2;
+    static constexpr int NQ = 2;  // 16 bf16 per lane
+    // v_mfma_f32_32x32x16_bf16: lane half h supplies 8 consecutive k of each 16-wide step;
+    // here step q contracts k in {8q..8q+7} u {16+8q..16+8q+7}.
+    static __device__ __forceinline__ void mma(f32x16& acc, const uint4* a, const uint4* b) {
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[q]),
+                                                          __builtin_bit_cast(bf16x8, b[q]), acc, 0, 0, 0);
+        }
+    }
+    // round to nearest even, NaN kept quiet
+    static __device__ __forceinline__ bf16_t from_f32(float v) {
+        uint32_t u = __float_as_uint(v);
+        bf16_t r;
+        if ((u & 0x7fffffffu) > 0x7f800000u) {
+            r.bits = (uint16_t)((u >> 16) | 0x40u);
+        } else {
+            u += 0x7fffu + ((u >> 16) & 1u);
+            r.bits = (uint16_t)(u >> 16);
+        }
+        return r;
+    }
+    static __device__ __forceinline__ float to_f32(bf16_t v) { return __uint_as_float(((uint32_t)v.bits) << 16); }
+};
+
+// Row of accumulator register v (0..15) held by a lane of half h in a 32x32 MFMA result;
+// the column is (lane & 31).
+static __device__ __forceinline__ int acc_row(int v, int h) { return 8 * (v >> 2) + 4 * h + (v & 3); }
+
+static __device__ __forceinline__ uint4 ldg16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
+
+// Two 16-byte rows of 8 bf16 (row k even, row k odd, same 8 columns) -> 8 words, word n holding
+// (row_even[n] low half, row_odd[n] high half): the k-pair packing the bf16 MFMA operands want.
+static __device__ __forceinline__ void interleave_bf16_rows(const uint4& r0, const uint4& r1, uint4& lo, uint4& hi) {
+    lo.x = (r0.x & 0xffffu) | (r1.x << 16);
+    lo.y = (r0.x >> 16) | (r1.x & 0xffff0000u);
+    lo.z = (r0.y & 0xffffu) | (r1.y << 16);
+    lo.w = (r0.y >> 16) | (r1.y & 0xffff0000u);
+    hi.x = (r0.z & 0xffffu) | (r1.z << 16);
+    hi.y = (r0.z >> 16) | (r1.z & 0xffff0000u);
+    hi.z = (r0.w & 0xffffu) | (r1.w << 16);
+    hi.w = (r0.w >> 16) | (r1.w & 0xffff0000u);
+}
+
+static constexpr int NUM_XCD = 8;
+
+// Workgroups are handed to the 8 XCDs round-robin by id.  Give each XCD one contiguous range of
+// logical tile ids, walked in launch order, so tiles that share an operand panel run on the same
+// XCD (one L2) at about the same time.  Returns -1 for the padding ids of the last range.
+static __device__ __forceinline__ int xcd_tile_id(int wg, int total) {
+    const int per = (total + NUM_XCD - 1) / NUM_XCD;
+    const int id = (wg % NUM_XCD) * per + wg / NUM_XCD;
+    return id < total ? id : -1;
+}
+static inline int xcd_grid(int total) { return ((total + NUM_XCD - 1) / NUM_XCD) * NUM_XCD; }
+
+}  // namespace pbs

@@ -1,0 +1,248 @@
+// C ABI of libpbs_hip.so: argument checks, tile-shape choice and kernel launches.
+#include "../../include/pbs_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+
+#include "pbs_common.h"
+#include "pbs_dds.h"
+#include "pbs_index.h"
+#include "pbs_sdd.h"
+
+namespace pbs {
+
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Zero fill as a kernel (callers may capture the stream into a graph).
+__global__ __launch_bounds__(256) void fill_zero_kernel(uint32_t* p, size_t nwords) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < nwords) p[i] = 0u;
+}
+
+// Kernels that use more than 64 KB of LDS need the limit raised once per device.
+template <typename K>
+static int raise_lds_limit(K kernel, int bytes, std::atomic<uint64_t>& done) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    const uint64_t bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return 0;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) return (int)e;
+    done.fetch_or(bit, std::memory_order_release);
+    return 0;
+}
+
+template <typename T, int TRANS, int TM, int TN, int WGM, int WGN>
+static int launch_dds(DdsArgs g, hipStream_t stream) {
+    using C = DdsCfg<T, TRANS, TM, TN, WGM, WGN>;
+    static std::atomic<uint64_t> done{0};
+    auto kernel = dds_kernel<T, TRANS, TM, TN, WGM, WGN>;
+    if (int rc = raise_lds_limit(kernel, C::LDS_BYTES, done)) return rc;
+    g.m_tiles = (g.M + C::BM - 1) / C::BM;
+    g.n_groups = (g.N / 32 + C::NB - 1) / C::NB;
+    const long long tiles = (long long)g.m_tiles * g.n_groups;
+    if (tiles > (1ll << 30)) return PBS_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)tiles)), dim3(C::NT), C::LDS_BYTES, stream, g);
+    return (int)hipGetLastError();
+}
+
+// Tile shapes.  fp32 is bound by the matrix cores long before LDS or the L1 fill path, so it
+// takes the smaller 128 x 128 tile (more workgroups, two per CU); bf16 issues 16x the flops per
+// staged byte and takes 256 tokens x 8 block columns with 8 waves.
+template <typename T, int TRANS>
+static int dispatch_dds(const DdsArgs& g, hipStream_t stream) {
+    if constexpr (sizeof(T) == 4) {
+        return launch_dds<T, TRANS, 2, 2, 2, 2>(g, stream);
+    } else {
+        const long long big_tiles = (long long)((g.M + 255) / 256) * ((g.N / 32 + 7) / 8);
+        if (big_tiles >= 256) return launch_dds<T, TRANS, 4, 2, 2, 4>(g, stream);
+        return launch_dds<T, TRANS, 2, 2, 2, 2>(g, stream);
+    }
+}
+
+// ---- sparse-output product ----
+template <typename T>
+struct SddShape;
+template <>
+struct SddShape<float> {
+    static constexpr int SR = 8, SC = 8, QW = 8, NW = 4;
+};
+template <>
+struct SddShape<bf16_t> {
+    static constexpr int SR = 8, SC = 16, QW = 8, NW = 8;
+};
+
+struct SddPlan {
+    int tiles_r, tiles_c, nsplit, tokens_per_split;
+};
+
+template <typename T>
+static SddPlan plan_sdd(long long M, int N, int K) {
+    using S = SddShape<T>;
+    using C = SddCfg<T, S::SR, S::SC, S::QW, S::NW>;
+    SddPlan p;
+    p.tiles_r = (N / 32 + S::SR - 1) / S::SR;
+    p.tiles_c = (K / 32 + S::SC - 1) / S::SC;
+    const long long tiles = (long long)p.tiles_r * p.tiles_c;
+    const long long chunks = (M + C::TC - 1) / C::TC;
+    // aim at two workgroups per CU, but keep at least 8 chunks of tokens per slice
+    long long want = (512 + tiles - 1) / tiles;
+    long long cap = chunks / 8;
+    if (cap < 1) cap = 1;
+    if (want > cap) want = cap;
+    if (want < 1) want = 1;
+    const long long chunks_per = (chunks + want - 1) / want;
+    p.nsplit = (int)((chunks + chunks_per - 1) / chunks_per);
+    if (p.nsplit < 1) p.nsplit = 1;
+    p.tokens_per_split = (int)(chunks_per * C::TC);
+    return p;
+}
+
+template <typename T>
+static int launch_sdd(SddArgs a, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    using S = SddShape<T>;
+    using C = SddCfg<T, S::SR, S::SC, S::QW, S::NW>;
+    static std::atomic<uint64_t> done{0};
+    auto kernel = sdd_kernel<T, S::SR, S::SC, S::QW, S::NW>;
+    if (int rc = raise_lds_limit(kernel, C::LDS_BYTES, done)) return rc;
+    const SddPlan p = plan_sdd<T>(a.M, a.N, a.K);
+    a.tiles_r = p.tiles_r;
+    a.tiles_c = p.tiles_c;
+    a.nsplit = p.nsplit;
+    a.tokens_per_split = p.tokens_per_split;
+    a.partial = nullptr;
+    const size_t n = (size_t)a.nnz * 1024;
+    if (p.nsplit > 1) {
+        const size_t need = n * sizeof(float) * p.nsplit;
+        if (!workspace || workspace_bytes < need || !aligned16(workspace)) return PBS_ERR_WORKSPACE;
+        a.partial = static_cast<float*>(workspace);
+    }
+    const long long wgs = (long long)p.tiles_r * p.tiles_c * p.nsplit;
+    if (wgs > (1ll << 30)) return PBS_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)wgs)), dim3(C::NT), C::LDS_BYTES, stream, a);
+    int rc = (int)hipGetLastError();
+    if (rc) return rc;
+    if (p.nsplit > 1) {
+        const unsigned grid = (unsigned)((n / 4 + 255) / 256);
+        hipLaunchKernelGGL(sdd_reduce_kernel<T>, dim3(grid), dim3(256), 0, stream, a.partial, static_cast<T*>(a.out), n,
+                           p.nsplit);
+        rc = (int)hipGetLastError();
+    }
+    return rc;
+}
+
+}  // namespace pbs
+
+using namespace pbs;
+
+extern "C" {
+
+int pbs_abi_version(void) { return PBS_ABI_VERSION; }
+
+const char* pbs_error_string(int code) {
+    switch (code) {
+        case PBS_OK: return "ok";
+        case PBS_ERR_NULL_POINTER: return "pbs: null pointer argument";
+        case PBS_ERR_BAD_SHAPE: return "pbs: bad shape (negative size, or a feature dimension that is not a multiple of 32)";
+        case PBS_ERR_BAD_DTYPE: return "pbs: unknown dtype code";
+        case PBS_ERR_MISALIGNED: return "pbs: dense/data pointers must be 16-byte aligned";
+        case PBS_ERR_WORKSPACE: return "pbs: workspace missing, misaligned or too small";
+        case PBS_ERR_TOO_LARGE: return "pbs: size exceeds the kernels' index range";
+        default: break;
+    }
+    if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
+    return "pbs: unknown error code";
+}
+
+int pbs_build_indices(const uint8_t* mask, const int64_t* block_ptr, int X, int Y, int nnz, int32_t* cols_a,
+                      int32_t* row_start_ends_a, int32_t* rows_b, int32_t* col_start_ends_b, int32_t* blocks,
+                      int32_t* status, void* stream) {
+    if (X < 1 || Y < 1 || nnz < 0 || (long long)nnz > (long long)X * Y) return PBS_ERR_BAD_SHAPE;
+    if ((long long)X * Y > (1ll << 30)) return PBS_ERR_TOO_LARGE;
+    if (!mask || !row_start_ends_a || !col_start_ends_b || !status) return PBS_ERR_NULL_POINTER;
+    if (nnz > 0 && (!cols_a || !rows_b || !blocks)) return PBS_ERR_NULL_POINTER;
+    hipLaunchKernelGGL(build_indices_kernel, dim3(1), dim3(INDEX_THREADS), 0, static_cast<hipStream_t>(stream), mask,
+                       block_ptr, X, Y, nnz, cols_a, row_start_ends_a, rows_b, col_start_ends_b, blocks, status);
+    return (int)hipGetLastError();
+}
+
+int pbs_blocksparse_matmul(const void* dense_a, const void* data, const int32_t* ptr, const int32_t* indices,
+                           const void* bias, void* dense_out, int64_t tokens, int n, int k, int nnz, int transpose,
+                           int dtype, void* stream) {
+    if (dtype != PBS_DTYPE_F32 && dtype != PBS_DTYPE_BF16) return PBS_ERR_BAD_DTYPE;
+    if (tokens < 0 || n <= 0 || k <= 0 || nnz < 0 || (n % 32) || (k % 32)) return PBS_ERR_BAD_SHAPE;
+    if (tokens > (1ll << 30) || (long long)nnz > (long long)(n / 32) * (k / 32)) return PBS_ERR_TOO_LARGE;
+    if (tokens == 0) return PBS_OK;
+    if (!dense_a || !ptr || !dense_out) return PBS_ERR_NULL_POINTER;
+    if (nnz > 0 && (!data || !indices)) return PBS_ERR_NULL_POINTER;
+    if (!aligned16(dense_a) || !aligned16(data)) return PBS_ERR_MISALIGNED;
+    DdsArgs g;
+    g.a = dense_a;
+    g.data = data;
+    g.ptr = ptr;
+    g.idx = indices;
+    g.bias = bias;
+    g.out = dense_out;
+    g.M = (int)tokens;
+    g.N = n;
+    g.K = k;
+    g.nnz = nnz;
+    g.m_tiles = g.n_groups = 0;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == PBS_DTYPE_F32) {
+        return transpose ? dispatch_dds<float, 0>(g, s) : dispatch_dds<float, 1>(g, s);
+    }
+    return transpose ? dispatch_dds<bf16_t, 0>(g, s) : dispatch_dds<bf16_t, 1>(g, s);
+}
+
+size_t pbs_blocksparse_matmul_back_workspace_bytes(int64_t tokens, int out_features, int in_features, int nnz,
+                                                   int dtype) {
+    if (tokens <= 0 || out_features <= 0 || in_features <= 0 || nnz <= 0) return 0;
+    if ((out_features % 32) || (in_features % 32)) return 0;
+    SddPlan p;
+    if (dtype == PBS_DTYPE_F32) p = plan_sdd<float>(tokens, out_features, in_features);
+    else if (dtype == PBS_DTYPE_BF16) p = plan_sdd<bf16_t>(tokens, out_features, in_features);
+    else return 0;
+    if (p.nsplit <= 1) return 0;
+    return (size_t)nnz * 1024 * sizeof(float) * p.nsplit;
+}
+
+int pbs_blocksparse_matmul_back(const void* dense_a, const void* dense_b, const int32_t* row_start_ends_a,
+                                const int32_t* cols_a, void* data_out, int64_t tokens, int out_features,
+                                int in_features, int nnz, int dtype, void* workspace, size_t workspace_bytes,
+                                void* stream) {
+    if (dtype != PBS_DTYPE_F32 && dtype != PBS_DTYPE_BF16) return PBS_ERR_BAD_DTYPE;
+    if (tokens < 0 || out_features <= 0 || in_features <= 0 || nnz < 0 || (out_features % 32) || (in_features % 32))
+        return PBS_ERR_BAD_SHAPE;
+    if (tokens > (1ll << 30) || (long long)nnz > (long long)(out_features / 32) * (in_features / 32))
+        return PBS_ERR_TOO_LARGE;
+    if (nnz == 0) return PBS_OK;
+    if (!row_start_ends_a || !cols_a || !data_out) return PBS_ERR_NULL_POINTER;
+    if (tokens > 0 && (!dense_a || !dense_b)) return PBS_ERR_NULL_POINTER;
+    if (!aligned16(dense_a) || !aligned16(dense_b) || !aligned16(data_out)) return PBS_ERR_MISALIGNED;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (tokens == 0) {
+        const size_t nwords = (size_t)nnz * 1024 * (dtype == PBS_DTYPE_F32 ? 4 : 2) / 4;
+        hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((nwords + 255) / 256)), dim3(256), 0, s,
+                           static_cast<uint32_t*>(data_out), nwords);
+        return (int)hipGetLastError();
+    }
+    SddArgs a;
+    a.g = dense_a;
+    a.x = dense_b;
+    a.ptr = row_start_ends_a;
+    a.idx = cols_a;
+    a.out = data_out;
+    a.partial = nullptr;
+    a.M = (int)tokens;
+    a.N = out_features;
+    a.K = in_features;
+    a.nnz = nnz;
+    a.tiles_r = a.tiles_c = a.nsplit = a.tokens_per_split = 0;
+    if (dtype == PBS_DTYPE_F32) return launch_sdd<float>(a, workspace, workspace_bytes, s);
+    return launch_sdd<bf16_t>(a, workspace, workspace_bytes, s);
+}
+
+}  // extern "C"

@@ -1,0 +1,313 @@
+// dense^T x dense -> block-sparse (weight gradient on the sparse support):
+//   out[32b + j][i] = sum_t G[t][32r + i] * X[t][32c + j]   for every data block b at (r, c).
+//
+// One workgroup owns an SR x SC rectangle of block positions of W and one slice of the tokens.
+// It lists the nonzero blocks inside its rectangle from the CSR arrays, deals them out to its
+// waves (at most QW accumulators each; more blocks than that are done in further passes), and
+// streams the tokens in chunks of TC: the chunk's G[TC, 32*SR] and X[TC, 32*SC] panels are
+// staged in LDS once, double buffered through registers, and shared by all blocks of the tile.
+// With more than one token slice the fp32 partial blocks go to a workspace and a second kernel
+// adds them in slice order, so the result does not depend on scheduling.
+#pragma once
+#include "pbs_common.h"
+
+namespace pbs {
+
+struct SddArgs {
+    const void* g;           // [M, N] grad_output, row-major
+    const void* x;           // [M, K] input, row-major
+    const int32_t* ptr;      // row_start_ends_a [N/32 + 1]
+    const int32_t* idx;      // cols_a [nnz][2] = (block col, data block)
+    void* out;               // [nnz*32, 32] (T) when nsplit == 1
+    float* partial;          // [nsplit][nnz*1024] fp32 when nsplit > 1
+    int M, N, K, nnz;
+    int tiles_r, tiles_c, nsplit;
+    int tokens_per_split;    // multiple of TC
+};
+
+template <typename T, int SR, int SC, int QW, int NW>
+struct SddCfg {
+    using E = Elem<T>;
+    static constexpr int NT = NW * 64;
+    static constexpr int TC = (E::ESZ == 4) ? 16 : 32;     // tokens per staged chunk
+    static constexpr int FG = SR * 32;                      // features per token row, G panel
+    static constexpr int FX = SC * 32;
+    // fp32: [t][f] words.  bf16: token pairs interleaved, [t/2][f] words of (t even, t odd).
+    static constexpr int ROWS = (E::ESZ == 4) ? TC : TC / 2;
+    static constexpr int G_BYTES = ROWS * FG * 4;
+    static constexpr int X_BYTES = ROWS * FX * 4;
+    static constexpr int STAGE_BYTES = G_BYTES + X_BYTES;
+    static constexpr int CG = TC * FG * E::ESZ / 16;        // 16-byte chunks per chunk of tokens
+    static constexpr int CX = TC * FX * E::ESZ / 16;
+    static constexpr int NG = CG / NT;
+    static constexpr int NX = CX / NT;
+    static constexpr int QMAX = QW * NW;
+    static constexpr int LIST_MAX = SR * SC;
+    static constexpr int LDS_BYTES = 2 * STAGE_BYTES + (LIST_MAX + SR + 4) * 4;
+    static_assert(CG % NT == 0 && CX % NT == 0, "staging must divide evenly");
+    static_assert(E::ESZ == 4 || (NG % 2 == 0 && NX % 2 == 0), "bf16 stages token pairs");
+    static_assert(SR <= 64 && SC <= 255 && SR <= 255, "list entry packs (rl, cl) in bytes");
+};
+
+template <typename T, int SR, int SC, int QW, int NW>
+__global__ __launch_bounds__(NW * 64) void sdd_kernel(SddArgs a) {
+    using C = SddCfg<T, SR, SC, QW, NW>;
+    using E = typename C::E;
+    constexpr int NT = C::NT, TC = C::TC, FG = C::FG, FX = C::FX;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    unsigned char* stage0 = smem;
+    int* s_list = reinterpret_cast<int*>(smem + 2 * C::STAGE_BYTES);  // (b << 12) | (rl << 8)... see pack
+    int* s_blk = s_list;                                               // [LIST_MAX] data block id
+    // the (rl, cl) pair of each listed block lives in a second array to keep ids full width
+    __shared__ unsigned short s_pos[C::LIST_MAX];
+    int* s_rowoff = s_list + C::LIST_MAX;                              // [SR+1]
+    __shared__ int s_count;
+
+    const int ntiles = a.tiles_r * a.tiles_c;
+    const int wg = xcd_tile_id(blockIdx.x, ntiles * a.nsplit);
+    if (wg < 0) return;
+    const int sp = wg / ntiles;            // token slice: slices of one tile land on different XCDs
+    const int tile = wg % ntiles;
+    const int tr = tile / a.tiles_c;
+    const int tc = tile % a.tiles_c;
+    const int r0 = tr * SR;
+    const int c0 = tc * SC;
+    const int nblk_r = a.N / 32;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int lrow = lane & 31;
+    const int h = lane >> 5;
+
+    // ---- list the nonzero blocks of the rectangle, row-major ----
+    int my_lo = 0, my_n = 0;
+    if (tid < SR) {
+        const int r = r0 + tid;
+        if (r < nblk_r) {
+            int lo = a.ptr[r], hi = a.ptr[r + 1];
+            // rows are sorted by block column: first entry with column >= c0
+            int l = lo, u = hi;
+            while (l < u) {
+                const int mid = (l + u) >> 1;
+                if (a.idx[2 * mid] < c0) l = mid + 1; else u = mid;
+            }
+            my_lo = l;
+            while (l < hi && a.idx[2 * l] < c0 + SC) ++l;
+            my_n = l - my_lo;
+        }
+        s_rowoff[tid] = my_n;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int run = 0;
+        for (int i = 0; i < SR; ++i) {
+            const int n = s_rowoff[i];
+            s_rowoff[i] = run;
+            run += n;
+        }
+        s_rowoff[SR] = run;
+        s_count = run;
+    }
+    __syncthreads();
+    if (tid < SR) {
+        const int off = s_rowoff[tid];
+        for (int i = 0; i < my_n; ++i) {
+            const int c = a.idx[2 * (my_lo + i)];
+            int b = a.idx[2 * (my_lo + i) + 1];
+            if (b < 0 || b >= a.nnz) b = -1;
+            s_blk[off + i] = b;
+            s_pos[off + i] = (unsigned short)((tid << 8) | (c - c0));
+        }
+    }
+    __syncthreads();
+    const int nq = s_count;
+    if (nq == 0) return;
+
+    const int t_begin = sp * a.tokens_per_split;
+    int t_end = t_begin + a.tokens_per_split;
+    if (t_end > a.M) t_end = a.M;
+    const int nchunks = t_begin < t_end ? (t_end - t_begin + TC - 1) / TC : 0;
+
+    const unsigned char* G = static_cast<const unsigned char*>(a.g);
+    const unsigned char* X = static_cast<const unsigned char*>(a.x);
+    const size_t g_col0 = (size_t)r0 * 32 * E::ESZ;
+    const size_t x_col0 = (size_t)c0 * 32 * E::ESZ;
+    const int g_valid = (a.N - r0 * 32) * E::ESZ;   // bytes of a G row that exist from column r0*32 on
+    const int x_valid = (a.K - c0 * 32) * E::ESZ;
+
+    uint4 rg[C::NG];
+    uint4 rx[C::NX];
+
+    // one 16-byte chunk of a panel: token row `t`, byte offset `cb` inside the panel's row
+    auto ld_panel = [&](const unsigned char* base, size_t ld_bytes, size_t col0, int valid, int t, int cb) -> uint4 {
+        if (t < t_end && cb < valid) return ldg16(base + (size_t)t * ld_bytes + col0 + cb);
+        return make_uint4(0, 0, 0, 0);
+    };
+    auto load_chunk = [&](int ci) {
+        const int t0 = t_begin + ci * TC;
+        if constexpr (E::ESZ == 4) {
+#pragma unroll
+            for (int i = 0; i < C::NG; ++i) {
+                const int q = i * NT + tid;
+                rg[i] = ld_panel(G, (size_t)a.N * 4, g_col0, g_valid, t0 + q / (FG / 4), (q % (FG / 4)) * 16);
+            }
+#pragma unroll
+            for (int i = 0; i < C::NX; ++i) {
+                const int q = i * NT + tid;
+                rx[i] = ld_panel(X, (size_t)a.K * 4, x_col0, x_valid, t0 + q / (FX / 4), (q % (FX / 4)) * 16);
+            }
+        } else {
+            // unit = (token pair, 8 features)
+#pragma unroll
+            for (int i = 0; i < C::NG / 2; ++i) {
+                const int u = i * NT + tid;
+                const int tp = u / (FG / 8), f8 = u % (FG / 8);
+                rg[2 * i] = ld_panel(G, (size_t)a.N * 2, g_col0, g_valid, t0 + 2 * tp, f8 * 16);
+                rg[2 * i + 1] = ld_panel(G, (size_t)a.N * 2, g_col0, g_valid, t0 + 2 * tp + 1, f8 * 16);
+            }
+#pragma unroll
+            for (int i = 0; i < C::NX / 2; ++i) {
+                const int u = i * NT + tid;
+                const int tp = u / (FX / 8), f8 = u % (FX / 8);
+                rx[2 * i] = ld_panel(X, (size_t)a.K * 2, x_col0, x_valid, t0 + 2 * tp, f8 * 16);
+                rx[2 * i + 1] = ld_panel(X, (size_t)a.K * 2, x_col0, x_valid, t0 + 2 * tp + 1, f8 * 16);
+            }
+        }
+    };
+    auto store_chunk = [&](int buf) {
+        unsigned char* sg = stage0 + buf * C::STAGE_BYTES;
+        unsigned char* sx = sg + C::G_BYTES;
+        if constexpr (E::ESZ == 4) {
+#pragma unroll
+            for (int i = 0; i < C::NG; ++i) reinterpret_cast<uint4*>(sg)[i * NT + tid] = rg[i];
+#pragma unroll
+            for (int i = 0; i < C::NX; ++i) reinterpret_cast<uint4*>(sx)[i * NT + tid] = rx[i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < C::NG / 2; ++i) {
+                const int u = i * NT + tid;
+                uint4 lo, hi;
+                interleave_bf16_rows(rg[2 * i], rg[2 * i + 1], lo, hi);
+                uint4* d = reinterpret_cast<uint4*>(sg) + 2 * u;   // [tp][f8*8 .. +7] words
+                d[0] = lo;
+                d[1] = hi;
+            }
+#pragma unroll
+            for (int i = 0; i < C::NX / 2; ++i) {
+                const int u = i * NT + tid;
+                uint4 lo, hi;
+                interleave_bf16_rows(rx[2 * i], rx[2 * i + 1], lo, hi);
+                uint4* d = reinterpret_cast<uint4*>(sx) + 2 * u;
+                d[0] = lo;
+                d[1] = hi;
+            }
+        }
+    };
+
+    T* out = static_cast<T*>(a.out);
+    float* part = a.partial ? a.partial + (size_t)sp * a.nnz * 1024 : nullptr;
+
+    for (int q0 = 0; q0 < nq; q0 += C::QMAX) {
+        // this pass: blocks [q0, q0 + npass), dealt to the waves in contiguous runs
+        const int npass = (nq - q0 < C::QMAX) ? nq - q0 : C::QMAX;
+        const int per = (npass + NW - 1) / NW;
+        const int w_lo = q0 + wave * per;
+        int w_n = q0 + npass - w_lo;
+        if (w_n > per) w_n = per;
+        if (w_n < 0) w_n = 0;
+
+        f32x16 acc[QW];
+#pragma unroll
+        for (int i = 0; i < QW; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
+
+        auto compute_chunk = [&](int buf) {
+            const uint32_t* sg = reinterpret_cast<const uint32_t*>(stage0 + buf * C::STAGE_BYTES);
+            const uint32_t* sx = reinterpret_cast<const uint32_t*>(stage0 + buf * C::STAGE_BYTES + C::G_BYTES);
+#pragma unroll
+            for (int i = 0; i < QW; ++i) {
+                if (i < w_n) {
+                    const int pos = __builtin_amdgcn_readfirstlane((int)s_pos[w_lo + i]);
+                    const int rl = pos >> 8, cl = pos & 255;
+                    const uint32_t* pa = sx + cl * 32 + lrow;   // A operand: X^T, rows = X feature j
+                    const uint32_t* pb = sg + rl * 32 + lrow;   // B operand: G,   cols = G feature i
+                    if constexpr (E::ESZ == 4) {
+                        // 16 tokens: lane half h holds tokens 8h .. 8h+7
+#pragma unroll
+                        for (int s = 0; s < 8; ++s) {
+                            const float av = __uint_as_float(pa[(8 * h + s) * FX]);
+                            const float bv = __uint_as_float(pb[(8 * h + s) * FG]);
+                            acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[i], 0, 0, 0);
+                        }
+                    } else {
+                        // 32 tokens = 16 pair rows: lane half h holds pair rows 8h .. 8h+7
+                        uint4 fa[2], fb[2];
+#pragma unroll
+                        for (int q = 0; q < 2; ++q) {
+                            fa[q].x = pa[(8 * h + 4 * q + 0) * FX];
+                            fa[q].y = pa[(8 * h + 4 * q + 1) * FX];
+                            fa[q].z = pa[(8 * h + 4 * q + 2) * FX];
+                            fa[q].w = pa[(8 * h + 4 * q + 3) * FX];
+                            fb[q].x = pb[(8 * h + 4 * q + 0) * FG];
+                            fb[q].y = pb[(8 * h + 4 * q + 1) * FG];
+                            fb[q].z = pb[(8 * h + 4 * q + 2) * FG];
+                            fb[q].w = pb[(8 * h + 4 * q + 3) * FG];
+                        }
+                        E::mma(acc[i], fa, fb);
+                    }
+                }
+            }
+        };
+
+        if (nchunks > 0) {
+            load_chunk(0);
+            store_chunk(0);
+            __syncthreads();
+            for (int ci = 0; ci < nchunks; ++ci) {
+                const bool more = ci + 1 < nchunks;
+                if (more) load_chunk(ci + 1);
+                compute_chunk(ci & 1);
+                if (more) store_chunk((ci + 1) & 1);
+                __syncthreads();
+            }
+        }
+
+        // ---- store: result row j (X feature), column i (G feature) ----
+#pragma unroll
+        for (int i = 0; i < QW; ++i) {
+            if (i < w_n) {
+                const int b = __builtin_amdgcn_readfirstlane(s_blk[w_lo + i]);
+                if (b >= 0) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const size_t o = (size_t)b * 1024 + acc_row(v, h) * 32 + lrow;
+                        if (part) part[o] = acc[i][v];
+                        else out[o] = E::from_f32(acc[i][v]);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// out[e] = sum over slices of partial[s][e], added in slice order.
+template <typename T>
+__global__ __launch_bounds__(256) void sdd_reduce_kernel(const float* partial, T* out, size_t n, int nsplit) {
+    using E = Elem<T>;
+    const size_t i4 = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i4 >= n) return;   // n is a multiple of 1024
+    float4 s = *reinterpret_cast<const float4*>(partial + i4);
+    for (int k = 1; k < nsplit; ++k) {
+        const float4 p = *reinterpret_cast<const float4*>(partial + (size_t)k * n + i4);
+        s.x += p.x; s.y += p.y; s.z += p.z; s.w += p.w;
+    }
+    out[i4 + 0] = E::from_f32(s.x);
+    out[i4 + 1] = E::from_f32(s.y);
+    out[i4 + 2] = E::from_f32(s.z);
+    out[i4 + 3] = E::from_f32(s.w);
+}
+
+}  // namespace pbs

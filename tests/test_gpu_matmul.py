@@ -1,0 +1,166 @@
+"""GPU parity of the three block-sparse matmuls against the dense-equivalent CPU oracle.
+
+Layouts and shapes follow the reference's tests/test_matmul.py (:141-244 tiny layouts, 1 token,
+3-D/4-D leading dims; :246-305 1024 -> 2048 at density 0.42 and 1.0) and tests/test_matmul_back.py
+(:205-277), plus the benchmark configurations.  Operands are signed N(0,1) (the reference uses
+positive operands so that isclose has no cancellation; here the absolute floor in assert_close
+plays that role).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import block_sparse_oracle as O
+from pytorch_block_sparse_amd import BlockSparseMatrix, workloads
+from tests.helpers import assert_close, to64
+
+pytestmark = pytest.mark.gpu
+
+TINY = [
+    # (lead dims of a, in_features, out_features, blocks)
+    ((32,), 32, 32, [(0, 0)]),
+    ((32,), 64, 32, [(0, 0)]),
+    ((64,), 32, 32, [(0, 0)]),
+    ((128,), 32, 32, [(0, 0)]),
+    ((128,), 64, 32, [(0, 0)]),
+    ((128,), 64, 32, [(0, 1)]),
+    ((128,), 64, 32, [(0, 0), (0, 1)]),
+    ((32,), 32, 64, [(0, 0)]),
+    ((32,), 32, 64, [(1, 0)]),
+    ((32,), 32, 64, [(0, 0), (1, 0)]),
+    ((64, 32), 32, 64, [(0, 0), (1, 0)]),
+    ((4, 8, 32), 128, 256, [(0, 0), (1, 0)]),
+    ((32,), 64, 64, [(0, 0), (1, 0), (0, 1)]),
+    ((32,), 64, 128, [(0, 0), (1, 0), (0, 1), (2, 0)]),
+    ((1,), 32, 32, [(0, 0)]),
+    ((1,), 64, 128, [(0, 0), (1, 0), (0, 1), (2, 0)]),
+    ((33,), 64, 128, [(0, 0), (1, 0), (0, 1), (2, 0)]),
+    ((77,), 96, 64, [(1, 2), (0, 0)]),
+]
+
+
+def _matrix(out_f, in_f, blocks, n_blocks, dtype, device, seed):
+    np.random.seed(seed)
+    torch.manual_seed(seed)
+    m = BlockSparseMatrix.randn((out_f, in_f), n_blocks, blocks=blocks, device="cpu", dtype=dtype)
+    return m.to(device)
+
+
+def _check_all(m, lead, dtype, device, seed, what):
+    out_f, in_f = m.shape
+    g = torch.Generator().manual_seed(seed + 1)
+    x = torch.randn(lead + (in_f,), generator=g).to(dtype)
+    dy = torch.randn(lead + (out_f,), generator=g).to(dtype)
+    coo = m.build_coo_block_index().cpu().numpy()
+    y_ref, dx_ref, dw_ref = O.linear_fwd_bwd(to64(x), to64(dy), to64(m.data), coo, tuple(m.shape))
+    xd, dyd = x.to(device), dy.to(device)
+    y = m.reverse_matmul(xd, transpose=True)
+    assert y.shape == lead + (out_f,)
+    assert_close(y, y_ref, dtype, what + " fwd")
+    dx = m.reverse_matmul(dyd, transpose=False)
+    assert dx.shape == lead + (in_f,)
+    assert_close(dx, dx_ref, dtype, what + " dx")
+    dw = m.matmul_with_output_sparse_support(dyd, xd)
+    assert dw.shape == m.data.shape
+    assert_close(dw, dw_ref, dtype, what + " dw")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_tiny_layouts(cuda, dtype):
+    for i, (lead, in_f, out_f, blocks) in enumerate(TINY):
+        print(f"tiny[{i}] lead={lead} {in_f}->{out_f} blocks={blocks} {dtype}", flush=True)
+        m = _matrix(out_f, in_f, blocks, None, dtype, cuda, seed=i)
+        _check_all(m, lead, dtype, cuda, i, f"tiny[{i}]")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("density", [0.42, 1.0, 0.05])
+@pytest.mark.parametrize("tokens", [1, 200, 1024])
+def test_1024_to_2048(cuda, dtype, density, tokens):
+    """reference: tests/test_matmul.py:246-305 shape (1024 -> 2048), tokens reduced to what the oracle does in seconds."""
+    print(f"1024->2048 d={density} tokens={tokens} {dtype}", flush=True)
+    n_blocks = int(density * 32 * 64)
+    m = _matrix(2048, 1024, None, n_blocks, dtype, cuda, seed=7)
+    _check_all(m, (tokens,), dtype, cuda, 11, f"d={density} t={tokens}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_empty_rows_and_columns(cuda, dtype):
+    """Block rows / columns without any block must come out as exact zeros (no pre-zeroed output)."""
+    m = _matrix(256, 192, [(1, 0), (1, 5), (6, 5)], None, dtype, cuda, seed=3)
+    x = torch.randn((100, 192), device=cuda).to(dtype)
+    y = m.reverse_matmul(x, transpose=True)
+    assert (y[:, :32] == 0).all() and (y[:, 64:192] == 0).all() and (y[:, 224:] == 0).all()
+    dy = torch.randn((100, 256), device=cuda).to(dtype)
+    dx = m.reverse_matmul(dy, transpose=False)
+    assert (dx[:, 32:160] == 0).all()
+    _check_all(m, (100,), dtype, cuda, 5, "empty rows")
+
+
+@pytest.mark.parametrize("name", ["c1_1024x256_d0.1_fp32", "c2_768x3072_d0.5_fp32", "c3_3072x768_d0.25_zipf_fp32"])
+def test_benchmark_configs_fp32(cuda, name):
+    w = workloads.WORKLOADS[name]
+    print(name, flush=True)
+    blocks, data, x, dy = workloads.make_inputs(w)
+    assert len(blocks) == w.nnz
+    m = BlockSparseMatrix.zeros((w.out_features, w.in_features), blocks=blocks, device="cpu", dtype=w.dtype)
+    with torch.no_grad():
+        # make_inputs lists blocks in row-major order, which is the data-block order
+        m.data.copy_(data)
+    m = m.to(cuda)
+    coo = m.build_coo_block_index().cpu().numpy()
+    y_ref, dx_ref, dw_ref = O.linear_fwd_bwd(to64(x), to64(dy), to64(data), coo, tuple(m.shape))
+    xd, dyd = x.to(cuda), dy.to(cuda)
+    assert_close(m.reverse_matmul(xd, True), y_ref, w.dtype, name + " fwd")
+    assert_close(m.reverse_matmul(dyd, False), dx_ref, w.dtype, name + " dx")
+    assert_close(m.matmul_with_output_sparse_support(dyd, xd), dw_ref, w.dtype, name + " dw")
+
+
+def test_benchmark_config_bf16_reduced_tokens(cuda):
+    """4096 -> 4096, density 0.25, bf16: oracle-checked on the first 2048 tokens of the workload."""
+    w = workloads.WORKLOADS["c4_4096x4096_d0.25_bf16"]
+    blocks, data, x, dy = workloads.make_inputs(w, tokens=2048)
+    m = BlockSparseMatrix.zeros((w.out_features, w.in_features), blocks=blocks, device="cpu", dtype=w.dtype)
+    with torch.no_grad():
+        m.data.copy_(data)
+    m = m.to(cuda)
+    coo = m.build_coo_block_index().cpu().numpy()
+    y_ref, dx_ref, dw_ref = O.linear_fwd_bwd(to64(x), to64(dy), to64(data), coo, tuple(m.shape))
+    xd, dyd = x.to(cuda), dy.to(cuda)
+    assert_close(m.reverse_matmul(xd, True), y_ref, w.dtype, "c4 fwd")
+    assert_close(m.reverse_matmul(dyd, False), dx_ref, w.dtype, "c4 dx")
+    assert_close(m.matmul_with_output_sparse_support(dyd, xd), dw_ref, w.dtype, "c4 dw")
+
+
+def test_benchmark_config_bf16_full_size_properties(cuda):
+    """Full 16384-token bf16 workload through size-independent properties.
+
+    * adjoint identity: <dY, X W^T> == <dY W, X> == <dW, W> (all three kernels tie together);
+    * token additivity of dW: dW(all tokens) == dW(first half) + dW(second half);
+    * row independence of fwd: rows of Y computed in the full call equal those of a 512-token call.
+    """
+    w = workloads.WORKLOADS["c4_4096x4096_d0.25_bf16"]
+    blocks, data, x, dy = workloads.make_inputs(w)
+    m = BlockSparseMatrix.zeros((w.out_features, w.in_features), blocks=blocks, device="cpu", dtype=w.dtype)
+    with torch.no_grad():
+        m.data.copy_(data)
+    m = m.to(cuda)
+    xd, dyd = x.to(cuda), dy.to(cuda)
+    y = m.reverse_matmul(xd, True)
+    dx = m.reverse_matmul(dyd, False)
+    dw = m.matmul_with_output_sparse_support(dyd, xd)
+    a = (dyd.double() * y.double()).sum().item()
+    b = (dx.double() * xd.double()).sum().item()
+    c = (dw.double() * m.data.double()).sum().item()
+    scale = (dyd.double().norm() * y.double().norm()).item()
+    print("adjoint", a, b, c, scale, flush=True)
+    # each side carries bf16 output rounding (2^-9 relative per element, random sign)
+    assert abs(a - b) < 2e-3 * scale and abs(a - c) < 2e-3 * scale
+    half = w.tokens // 2
+    dw1 = m.matmul_with_output_sparse_support(dyd[:half], xd[:half])
+    dw2 = m.matmul_with_output_sparse_support(dyd[half:], xd[half:])
+    ref = dw1.double() + dw2.double()
+    err = (dw.double() - ref).abs().max().item()
+    assert err < 3 * 2.0 ** -8 * ref.abs().max().item(), err
+    y_small = m.reverse_matmul(xd[1024:1536], True)
+    assert torch.equal(y_small, y[1024:1536])
