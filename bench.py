@@ -1,0 +1,210 @@
+#!/usr/bin/env python3
+"""Benchmark of the block-sparse linear hot path on one MI355X.
+
+One step = forward Y = X.W^T, input gradient dX = dY.W and weight gradient dW = dY^T.X on the
+sparse support, for BlockSparseLinear(4096 -> 4096, density 0.25), 16384 tokens, bf16 operands
+with fp32 accumulation.  Inputs are synthetic (seeded) and resident in HBM before timing starts.
+
+Prints ONE JSON line: effective TFLOP/s (2*M*nnz*1024 per GEMM, 3 GEMMs per step) with
+  roofline      the slowest of the three kernels against the MI355X dense bf16 MFMA peak,
+  dense         the same three GEMMs dense through torch.matmul (hipBLASLt) at the same shape,
+  cpu_baseline  the CPU dense-equivalent path (oracle) timed on the host cores on a token sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}  # MI355X dense matrix peaks
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=50)
+    p.add_argument("--warmup", type=int, default=10)
+    p.add_argument("--workload", default="c4_4096x4096_d0.25_bf16")
+    p.add_argument("--tokens", type=int, default=None, help="override the workload's token count")
+    p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    p.add_argument("--no-dense", action="store_true", help="skip the dense hipBLASLt leg")
+    p.add_argument("--cpu-sample-tokens", type=int, default=2048)
+    return p.parse_args()
+
+
+def time_gpu(fn, steps, warmup):
+    """Average milliseconds per call of fn over `steps` calls, HIP events on the current stream."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / steps
+
+
+def cpu_baseline(w, sample_tokens):
+    """The reference's CPU dense-equivalent path (to_dense + matmul, fp32) on the first sample_tokens tokens."""
+    import torch
+
+    from oracle import block_sparse_oracle as O
+    from pytorch_block_sparse_amd import workloads
+
+    blocks, data, x, dy = workloads.make_inputs(w, tokens=sample_tokens)
+    X, Y = w.grid
+    mask = O.mask_from_blocks(X, Y, blocks)
+    idx = O.build_indices(mask)
+    coo = O.build_coo_block_index(idx["row_start_ends_a"], idx["cols_a"])
+    shape = (w.out_features, w.in_features)
+    w_dense = torch.from_numpy(O.to_dense(data.float().numpy(), coo, shape))
+    mask_dense = torch.from_numpy(O.block_mask_dense(coo, shape)).float()
+    xf, dyf = x.float(), dy.float()
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    O.linear_fwd_bwd_torch_fp32(xf, dyf, w_dense, mask_dense)  # warm-up
+    times = []
+    t_all = time.perf_counter()
+    while len(times) < 5 and (len(times) < 2 or time.perf_counter() - t_all < 20.0):
+        t0 = time.perf_counter()
+        O.linear_fwd_bwd_torch_fp32(xf, dyf, w_dense, mask_dense)
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    eff = 3 * 2.0 * sample_tokens * w.nnz * 1024 / med / 1e12
+    return {
+        "value": eff,
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"first {sample_tokens} of {w.tokens} tokens, same layer; torch CPU fp32 dense-equivalent "
+        f"fwd+dX+dW, median of {len(times)} runs ({med * 1e3:.1f} ms)",
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only; --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from pytorch_block_sparse_amd import BlockSparseMatrix, native, workloads
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    native.load()  # fail loudly if the HIP library is not built
+    dev = torch.device("cuda:0")
+    w = workloads.WORKLOADS[args.workload]
+    tokens = args.tokens or w.tokens
+    blocks, data, x, dy = workloads.make_inputs(w, tokens=tokens)
+    m = BlockSparseMatrix.zeros((w.out_features, w.in_features), blocks=blocks, device="cpu", dtype=w.dtype)
+    with torch.no_grad():
+        m.data.copy_(data)
+    m = m.to(dev)
+    xd, dyd = x.to(dev), dy.to(dev)
+    torch.cuda.synchronize()
+
+    def fwd():
+        return m.reverse_matmul(xd, True)
+
+    def dx():
+        return m.reverse_matmul(dyd, False)
+
+    def dw():
+        return m.matmul_with_output_sparse_support(dyd, xd)
+
+    if w.passes == "fwd":
+        kernels = {"fwd": fwd}
+    else:
+        kernels = {"fwd": fwd, "dx": dx, "dw": dw}
+
+    def step():
+        for f in kernels.values():
+            f()
+
+    ms_step = time_gpu(step, args.steps, args.warmup)
+    per_kernel = {k: time_gpu(f, args.steps, min(args.warmup, 3)) for k, f in kernels.items()}
+
+    dname = "bf16" if w.dtype == torch.bfloat16 else "f32"
+    flops_gemm = 2.0 * tokens * w.nnz * 1024
+    n_gemms = len(kernels)
+    value = n_gemms * flops_gemm / (ms_step * 1e-3) / 1e12
+    dom = max(per_kernel, key=per_kernel.get)
+    achieved = flops_gemm / (per_kernel[dom] * 1e-3) / 1e12
+    kernel_names = {"fwd": "dds_kernel<TRANS=0>", "dx": "dds_kernel<TRANS=1>", "dw": "sdd_kernel(+sdd_reduce_kernel)"}
+
+    out = {
+        "metric": "effective TFLOP/s fwd+bwd at 4096^2 d=0.25; % of MFMA peak; vs dense GEMM",
+        "value": value,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dname,
+        "data": "synthetic",
+        "config": {
+            "workload": w.name,
+            "in_features": w.in_features,
+            "out_features": w.out_features,
+            "density": w.density,
+            "nnz_blocks": w.nnz,
+            "tokens": tokens,
+            "pattern": w.pattern,
+            "passes": w.passes,
+        },
+        "pct_of_mfma_peak": 100.0 * value / PEAK_TFLOPS[dname],
+        "kernel_ms": per_kernel,
+        "kernel_eff_tflops": {k: flops_gemm / (v * 1e-3) / 1e12 for k, v in per_kernel.items()},
+        "roofline": {
+            "bound": "mfma",
+            "kernel": kernel_names[dom],
+            "achieved": achieved,
+            "peak": PEAK_TFLOPS[dname],
+            "unit": "TFLOP/s",
+            "frac": achieved / PEAK_TFLOPS[dname],
+            "traffic": None,
+        },
+    }
+
+    if not args.no_dense:
+        wd = m.to_dense()
+        dense = {
+            "fwd": lambda: xd @ wd.t(),
+            "dx": lambda: dyd @ wd,
+            "dw": lambda: dyd.t() @ xd,
+        }
+        if w.passes == "fwd":
+            dense = {"fwd": dense["fwd"]}
+
+        def dense_step():
+            for f in dense.values():
+                f()
+
+        ms_dense = time_gpu(dense_step, args.steps, args.warmup)
+        out["dense_hipblaslt"] = {
+            "ms_per_step": ms_dense,
+            "dense_tflops": n_gemms * 2.0 * tokens * w.in_features * w.out_features / (ms_dense * 1e-3) / 1e12,
+            "speedup_sparse_vs_dense": ms_dense / ms_step,
+        }
+        del wd
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(w, min(args.cpu_sample_tokens, tokens))
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
