@@ -87,6 +87,15 @@ static __device__ __forceinline__ void interleave_bf16_rows(const uint4& r0, con
     hi.w = (r0.w >> 16) | (r1.w & 0xffff0000u);
 }
 
+// ds_read_b64_tr_b16: within each group of 16 lanes, lane s passes the LDS address of 4 consecutive
+// 16-bit elements (row s/4 of a 4 x 16 tile, columns 4*(s%4)..+3) and lane j receives column j of
+// the tile: the 4 rows' elements, in row order.
+static __device__ __forceinline__ uint2 tr16_b64(const unsigned char* lds_ptr) {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(lds_ptr));
+    return __builtin_bit_cast(uint2, v);
+}
+
 static constexpr int NUM_XCD = 8;
 
 // Workgroups are handed to the 8 XCDs round-robin by id.  Give each XCD one contiguous range of

@@ -34,31 +34,32 @@ static int raise_lds_limit(K kernel, int bytes, std::atomic<uint64_t>& done) {
     return 0;
 }
 
-template <typename T, int TRANS, int TM, int TN, int WGM, int WGN>
+template <typename T, int TRANS, int TM, int NB, int NW, int SK, int RS, int RB>
 static int launch_dds(DdsArgs g, hipStream_t stream) {
-    using C = DdsCfg<T, TRANS, TM, TN, WGM, WGN>;
+    using C = DdsCfg<T, TRANS, TM, NB, NW, SK, RS, RB>;
     static std::atomic<uint64_t> done{0};
-    auto kernel = dds_kernel<T, TRANS, TM, TN, WGM, WGN>;
+    auto kernel = dds_kernel<T, TRANS, TM, NB, NW, SK, RS, RB>;
     if (int rc = raise_lds_limit(kernel, C::LDS_BYTES, done)) return rc;
     g.m_tiles = (g.M + C::BM - 1) / C::BM;
-    g.n_groups = (g.N / 32 + C::NB - 1) / C::NB;
+    g.n_groups = (g.N / 32 + NB - 1) / NB;
     const long long tiles = (long long)g.m_tiles * g.n_groups;
     if (tiles > (1ll << 30)) return PBS_ERR_TOO_LARGE;
     hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)tiles)), dim3(C::NT), C::LDS_BYTES, stream, g);
     return (int)hipGetLastError();
 }
 
-// Tile shapes.  fp32 is bound by the matrix cores long before LDS or the L1 fill path, so it
-// takes the smaller 128 x 128 tile (more workgroups, two per CU); bf16 issues 16x the flops per
-// staged byte and takes 256 tokens x 8 block columns with 8 waves.
+// Tile shapes: 4 waves that split the tokens, 8 block columns per workgroup (256 x 256 results)
+// when that still gives every CU a tile, else 128 tokens x 4 block columns.  bf16 steps cover two
+// k-blocks (the matrix cores go through a k-block 16x faster than in fp32).
 template <typename T, int TRANS>
 static int dispatch_dds(const DdsArgs& g, hipStream_t stream) {
+    const long long big_tiles = (long long)((g.M + 255) / 256) * ((g.N / 32 + 7) / 8);
     if constexpr (sizeof(T) == 4) {
-        return launch_dds<T, TRANS, 2, 2, 2, 2>(g, stream);
+        if (big_tiles >= 256) return launch_dds<T, TRANS, 2, 8, 4, 1, 3, 8>(g, stream);
+        return launch_dds<T, TRANS, 1, 4, 4, 1, 3, 8>(g, stream);
     } else {
-        const long long big_tiles = (long long)((g.M + 255) / 256) * ((g.N / 32 + 7) / 8);
-        if (big_tiles >= 256) return launch_dds<T, TRANS, 4, 2, 2, 4>(g, stream);
-        return launch_dds<T, TRANS, 2, 2, 2, 2>(g, stream);
+        if (big_tiles >= 256) return launch_dds<T, TRANS, 2, 8, 4, 2, 3, 16>(g, stream);
+        return launch_dds<T, TRANS, 1, 4, 4, 2, 4, 8>(g, stream);
     }
 }
 
