@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define PBS_ABI_VERSION 1
+#define PBS_ABI_VERSION 2
 #define PBS_BLOCK 32
 
 /* element type of dense operands, packed data and results (accumulation is fp32) */
@@ -42,7 +42,7 @@ extern "C" {
 #define PBS_ERR_BAD_SHAPE (-2)     /* negative size or a feature dim not a multiple of 32 */
 #define PBS_ERR_BAD_DTYPE (-3)
 #define PBS_ERR_MISALIGNED (-4)    /* a dense/data pointer is not 16-byte aligned */
-#define PBS_ERR_WORKSPACE (-5)     /* workspace missing or smaller than pbs_*_workspace_bytes */
+#define PBS_ERR_WORKSPACE (-5)     /* workspace/plan buffer missing, misaligned or too small */
 #define PBS_ERR_TOO_LARGE (-6)     /* a size exceeds what the kernels index with */
 
 int pbs_abi_version(void);
@@ -66,24 +66,39 @@ int pbs_build_indices(const uint8_t* mask, const int64_t* block_ptr, int X, int 
                       int32_t* blocks, int32_t* status, void* stream);
 
 /*
+ * Schedule ("plan") of the dense x block-sparse product for one pattern and one direction.
+ * It depends only on the index arrays, not on the data: build it when the pattern is created or
+ * changed and pass it to every pbs_blocksparse_matmul call of that direction.  It is what the
+ * reference's kernel derives again in every thread block from ptr/indices
+ * (cutlass/gemm/block_loader_crosswise_prune_dense.h:254-264, :398-444), hoisted out of the hot
+ * path: per group of 8 result block columns, the merged list of k-blocks they touch.
+ *
+ *   transpose = 1 (forward):        ptr = row_start_ends_a, indices = cols_a, n = out, k = in
+ *   transpose = 0 (input gradient): ptr = col_start_ends_b, indices = rows_b, n = in,  k = out
+ *   plan: 16-byte aligned device buffer of pbs_blocksparse_matmul_plan_bytes(n, k) bytes
+ */
+size_t pbs_blocksparse_matmul_plan_bytes(int n, int k);
+int pbs_blocksparse_matmul_plan(const int32_t* ptr, const int32_t* indices, int n, int k, int nnz,
+                                void* plan, size_t plan_bytes, void* stream);
+
+/*
  * dense x block-sparse -> dense.  Replaces blocksparse_matmul_cutlass
  * (native/block_sparse_native.cpp:6-16, launcher native/block_sparse_cutlass_kernel.cu:113-150)
  * as called by BlockSparseMatrixBase.reverse_matmul_ (block_sparse.py:496-578).
  *
- *   transpose = 1 : out[tokens, n] = a[tokens, k] . W^T   n = out_features, k = in_features,
- *                   ptr = row_start_ends_a, indices = cols_a          (forward, :518-521)
- *   transpose = 0 : out[tokens, n] = a[tokens, k] . W     n = in_features,  k = out_features,
- *                   ptr = col_start_ends_b, indices = rows_b          (input gradient, :522-525)
+ *   transpose = 1 : out[tokens, n] = a[tokens, k] . W^T   n = out_features, k = in_features  (:518-521)
+ *   transpose = 0 : out[tokens, n] = a[tokens, k] . W     n = in_features,  k = out_features (:522-525)
+ *   plan: built by pbs_blocksparse_matmul_plan from the (ptr, indices) pair the reference passes
+ *         here, for the same transpose
  *
- * Differences from the reference entry point, all on purpose: `data` is always the
- * packed data as stored (no per-call transposed copy of the weights, :541-544); `out`
- * is row-major [tokens, n] and need not be zeroed (the reference wants a zeroed
- * [n, tokens] buffer, :516); `bias` is NULL or [n] and is added in the epilogue
- * (the reference adds it in a separate pass, block_sparse_linear.py:231-232);
- * any tokens >= 0 is handled; work is launched on `stream`, not on stream 0.
+ * Differences from the reference entry point, all on purpose: `data` is always the packed data as
+ * stored (no per-call transposed copy of the weights, :541-544); `out` is row-major [tokens, n]
+ * and need not be zeroed (the reference wants a zeroed [n, tokens] buffer, :516); `bias` is NULL
+ * or [n] and is added in the epilogue (the reference adds it in a separate pass,
+ * block_sparse_linear.py:231-232); any tokens >= 0 is handled; work is launched on `stream`,
+ * not on stream 0.
  */
-int pbs_blocksparse_matmul(const void* dense_a, const void* data,
-                           const int32_t* ptr, const int32_t* indices,
+int pbs_blocksparse_matmul(const void* dense_a, const void* data, const void* plan,
                            const void* bias, void* dense_out,
                            int64_t tokens, int n, int k, int nnz,
                            int transpose, int dtype, void* stream);

@@ -86,6 +86,7 @@ class BlockSparseMatrixBase(torch.nn.Module):
         self.register_buffer("rows_b", rows_b)
         self.register_buffer("col_start_ends_b", col_start_ends_b)
         self.register_buffer("blocks", blocks)
+        self._plans = {}
         self.check_ = False
         if callback:
             self.updated_data()
@@ -365,15 +366,27 @@ class BlockSparseMatrixBase(torch.nn.Module):
         k, n = (cols, rows) if transpose else (rows, cols)
         if dense_a.shape[1] != k:
             raise Exception("Invalid matrices sizes (%d, %d) x (%d, %d)" % (dense_a.shape[0], dense_a.shape[1], k, n))
-        if transpose:
-            ptr, indices = self.row_start_ends_a, self.cols_a
-        else:
-            ptr, indices = self.col_start_ends_b, self.rows_b
         dense_a = self.tensor_prepare(dense_a)
         data = self.data.detach()
         if not data.is_contiguous():
             raise Exception("block data must be contiguous")
-        return native.blocksparse_matmul(dense_a, data, ptr, indices, n, k, transpose, bias=bias)
+        plan = self._matmul_plan(bool(transpose), n, k)
+        return native.blocksparse_matmul(dense_a, data, plan, n, k, self.cols_a.shape[0], transpose, bias=bias)
+
+    def _matmul_plan(self, transpose, n, k):
+        """Kernel schedule of this pattern for one direction, built on first use and kept until the
+        index buffers change (rebuild, load_state_dict, move to another device)."""
+        if transpose:
+            ptr, indices = self.row_start_ends_a, self.cols_a
+        else:
+            ptr, indices = self.col_start_ends_b, self.rows_b
+        plans = self.__dict__.setdefault("_plans", {})
+        key = (transpose, ptr.data_ptr(), indices.data_ptr(), ptr._version, indices._version)
+        hit = plans.get(transpose)
+        if hit is None or hit[0] != key:
+            hit = (key, native.blocksparse_matmul_plan(ptr, indices, n, k))
+            plans[transpose] = hit
+        return hit[1]
 
     def reverse_matmul(self, dense_a, transpose, bias=None):
         """Any leading dims.  reference: block_sparse.py:597-604."""

@@ -34,32 +34,34 @@ static int raise_lds_limit(K kernel, int bytes, std::atomic<uint64_t>& done) {
     return 0;
 }
 
-template <typename T, int TRANS, int TM, int NB, int NW, int SK, int RS, int RB>
+template <typename T, int TRANS, int TM, int SK, int RS, int RB, int NP>
 static int launch_dds(DdsArgs g, hipStream_t stream) {
-    using C = DdsCfg<T, TRANS, TM, NB, NW, SK, RS, RB>;
+    using C = DdsCfg<T, TRANS, TM, SK, RS, RB, NP>;
     static std::atomic<uint64_t> done{0};
-    auto kernel = dds_kernel<T, TRANS, TM, NB, NW, SK, RS, RB>;
+    auto kernel = dds_kernel<T, TRANS, TM, SK, RS, RB, NP>;
     if (int rc = raise_lds_limit(kernel, C::LDS_BYTES, done)) return rc;
     g.m_tiles = (g.M + C::BM - 1) / C::BM;
-    g.n_groups = (g.N / 32 + NB - 1) / NB;
     const long long tiles = (long long)g.m_tiles * g.n_groups;
     if (tiles > (1ll << 30)) return PBS_ERR_TOO_LARGE;
     hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)tiles)), dim3(C::NT), C::LDS_BYTES, stream, g);
     return (int)hipGetLastError();
 }
 
-// Tile shapes: 4 waves that split the tokens, 8 block columns per workgroup (256 x 256 results)
-// when that still gives every CU a tile, else 128 tokens x 4 block columns.  bf16 steps cover two
-// k-blocks (the matrix cores go through a k-block 16x faster than in fp32).
+// Tile shapes: 256 tokens x 8 block columns when that still gives every CU a tile, else 128 tokens.
+// bf16 steps cover two k-blocks (the matrix cores go through a k-block 16x faster than in fp32).
 template <typename T, int TRANS>
 static int dispatch_dds(const DdsArgs& g, hipStream_t stream) {
-    const long long big_tiles = (long long)((g.M + 255) / 256) * ((g.N / 32 + 7) / 8);
+    const long long big_tiles = (long long)((g.M + 255) / 256) * g.n_groups;
     if constexpr (sizeof(T) == 4) {
-        if (big_tiles >= 256) return launch_dds<T, TRANS, 2, 8, 4, 1, 3, 8>(g, stream);
-        return launch_dds<T, TRANS, 1, 4, 4, 1, 3, 8>(g, stream);
+        if (big_tiles >= 256) return launch_dds<T, TRANS, 2, 1, 3, 8, 0>(g, stream);
+        return launch_dds<T, TRANS, 1, 1, 3, 8, 0>(g, stream);
     } else {
-        if (big_tiles >= 256) return launch_dds<T, TRANS, 2, 8, 4, 2, 3, 16>(g, stream);
-        return launch_dds<T, TRANS, 1, 4, 4, 2, 4, 8>(g, stream);
+#ifdef PBS_EXP_BF16_CFG
+        return launch_dds<T, TRANS, PBS_EXP_BF16_CFG>(g, stream);
+#else
+        if (big_tiles >= 256) return launch_dds<T, TRANS, 2, 2, 3, 16, 4>(g, stream);
+        return launch_dds<T, TRANS, 1, 2, 3, 16, 4>(g, stream);
+#endif
     }
 }
 
@@ -142,6 +144,13 @@ extern "C" {
 
 int pbs_abi_version(void) { return PBS_ABI_VERSION; }
 
+#ifdef PBS_EXP_TIMING
+int pbs_debug_read_prof(long long* host, int n) {
+    hipDeviceSynchronize();
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_prof), (size_t)n * 8);
+}
+#endif
+
 const char* pbs_error_string(int code) {
     switch (code) {
         case PBS_OK: return "ok";
@@ -169,28 +178,46 @@ int pbs_build_indices(const uint8_t* mask, const int64_t* block_ptr, int X, int 
     return (int)hipGetLastError();
 }
 
-int pbs_blocksparse_matmul(const void* dense_a, const void* data, const int32_t* ptr, const int32_t* indices,
-                           const void* bias, void* dense_out, int64_t tokens, int n, int k, int nnz, int transpose,
-                           int dtype, void* stream) {
+size_t pbs_blocksparse_matmul_plan_bytes(int n, int k) {
+    if (n <= 0 || k <= 0 || (n % 32) || (k % 32)) return 0;
+    const size_t groups = ((size_t)(n / 32) + DDS_NB - 1) / DDS_NB;
+    return groups * dds_plan_group_ints(k / 32) * sizeof(int);
+}
+
+int pbs_blocksparse_matmul_plan(const int32_t* ptr, const int32_t* indices, int n, int k, int nnz, void* plan,
+                                size_t plan_bytes, void* stream) {
+    if (n <= 0 || k <= 0 || nnz < 0 || (n % 32) || (k % 32)) return PBS_ERR_BAD_SHAPE;
+    if ((long long)nnz > (long long)(n / 32) * (k / 32) || k > (1 << 24)) return PBS_ERR_TOO_LARGE;
+    if (!ptr || !plan || (nnz > 0 && !indices)) return PBS_ERR_NULL_POINTER;
+    if (!aligned16(plan) || plan_bytes < pbs_blocksparse_matmul_plan_bytes(n, k)) return PBS_ERR_WORKSPACE;
+    const int groups = (n / 32 + DDS_NB - 1) / DDS_NB;
+    hipLaunchKernelGGL(dds_plan_kernel, dim3(groups), dim3(256), 0, static_cast<hipStream_t>(stream), ptr, indices, n / 32,
+                       k / 32, nnz, static_cast<int*>(plan), (int)dds_plan_group_ints(k / 32));
+    return (int)hipGetLastError();
+}
+
+int pbs_blocksparse_matmul(const void* dense_a, const void* data, const void* plan, const void* bias, void* dense_out,
+                           int64_t tokens, int n, int k, int nnz, int transpose, int dtype, void* stream) {
     if (dtype != PBS_DTYPE_F32 && dtype != PBS_DTYPE_BF16) return PBS_ERR_BAD_DTYPE;
     if (tokens < 0 || n <= 0 || k <= 0 || nnz < 0 || (n % 32) || (k % 32)) return PBS_ERR_BAD_SHAPE;
-    if (tokens > (1ll << 30) || (long long)nnz > (long long)(n / 32) * (k / 32)) return PBS_ERR_TOO_LARGE;
+    if (tokens > (1ll << 30) || (long long)nnz > (long long)(n / 32) * (k / 32) || k > (1 << 24)) return PBS_ERR_TOO_LARGE;
     if (tokens == 0) return PBS_OK;
-    if (!dense_a || !ptr || !dense_out) return PBS_ERR_NULL_POINTER;
-    if (nnz > 0 && (!data || !indices)) return PBS_ERR_NULL_POINTER;
-    if (!aligned16(dense_a) || !aligned16(data)) return PBS_ERR_MISALIGNED;
+    if (!dense_a || !plan || !dense_out) return PBS_ERR_NULL_POINTER;
+    if (nnz > 0 && !data) return PBS_ERR_NULL_POINTER;
+    if (!aligned16(dense_a) || !aligned16(data) || !aligned16(dense_out) || !aligned16(plan)) return PBS_ERR_MISALIGNED;
     DdsArgs g;
     g.a = dense_a;
     g.data = data;
-    g.ptr = ptr;
-    g.idx = indices;
+    g.plan = static_cast<const int*>(plan);
     g.bias = bias;
     g.out = dense_out;
     g.M = (int)tokens;
     g.N = n;
     g.K = k;
     g.nnz = nnz;
-    g.m_tiles = g.n_groups = 0;
+    g.m_tiles = 0;
+    g.n_groups = (n / 32 + DDS_NB - 1) / DDS_NB;
+    g.group_ints = (int)dds_plan_group_ints(k / 32);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == PBS_DTYPE_F32) {
         return transpose ? dispatch_dds<float, 0>(g, s) : dispatch_dds<float, 1>(g, s);

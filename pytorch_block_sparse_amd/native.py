@@ -30,7 +30,9 @@ _PROTOTYPES = {
     "pbs_abi_version": (ctypes.c_int, []),
     "pbs_error_string": (ctypes.c_char_p, [_i32]),
     "pbs_build_indices": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
-    "pbs_blocksparse_matmul": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _vp]),
+    "pbs_blocksparse_matmul_plan_bytes": (ctypes.c_size_t, [_i32, _i32]),
+    "pbs_blocksparse_matmul_plan": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp, ctypes.c_size_t, _vp]),
+    "pbs_blocksparse_matmul": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _vp]),
     "pbs_blocksparse_matmul_back_workspace_bytes": (ctypes.c_size_t, [_i64, _i32, _i32, _i32, _i32]),
     "pbs_blocksparse_matmul_back": (
         _i32,
@@ -124,10 +126,24 @@ def build_indices(block_mask, block_ptr, nnz):
     return blocks, cols_a, row_ptr, rows_b, col_ptr
 
 
-def blocksparse_matmul(dense_a, data, ptr, indices, n, k, transpose, bias=None, out=None):
+def blocksparse_matmul_plan(ptr, indices, n, k):
+    """Schedule buffer of the dense x block-sparse product for (ptr, indices); depends on the pattern only."""
+    lib = load()
+    _require_cuda(ptr, indices)
+    nbytes = lib.pbs_blocksparse_matmul_plan_bytes(n, k)
+    plan = torch.empty((nbytes // 4,), dtype=torch.int32, device=ptr.device)
+    with torch.cuda.device(ptr.device):
+        code = lib.pbs_blocksparse_matmul_plan(
+            _ptr(ptr), _ptr(indices), n, k, indices.shape[0], _ptr(plan), nbytes, _stream()
+        )
+    _check(code, "pbs_blocksparse_matmul_plan")
+    return plan
+
+
+def blocksparse_matmul(dense_a, data, plan, n, k, nnz, transpose, bias=None, out=None):
     """out[tokens, n] = dense_a[tokens, k] . W^T (transpose) or . W (not transpose)."""
     lib = load()
-    _require_cuda(dense_a, data, ptr, indices, bias)
+    _require_cuda(dense_a, data, plan, bias)
     if dense_a.dtype not in DTYPE_CODES:
         raise RuntimeError(f"unsupported dtype {dense_a.dtype}; supported: {SUPPORTED_DTYPES}")
     if data.dtype != dense_a.dtype:
@@ -137,10 +153,9 @@ def blocksparse_matmul(dense_a, data, ptr, indices, n, k, transpose, bias=None, 
     tokens = dense_a.shape[0]
     if out is None:
         out = torch.empty((tokens, n), dtype=dense_a.dtype, device=dense_a.device)
-    nnz = indices.shape[0]
     with torch.cuda.device(dense_a.device):
         code = lib.pbs_blocksparse_matmul(
-            _ptr(dense_a), _ptr(data), _ptr(ptr), _ptr(indices), _ptr(bias), _ptr(out), tokens, n, k, nnz,
+            _ptr(dense_a), _ptr(data), _ptr(plan), _ptr(bias), _ptr(out), tokens, n, k, nnz,
             1 if transpose else 0, DTYPE_CODES[dense_a.dtype], _stream(),
         )
     _check(code, "pbs_blocksparse_matmul")
