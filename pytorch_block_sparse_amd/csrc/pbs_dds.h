@@ -1,28 +1,28 @@
 // dense x block-sparse -> dense (forward Y = X.W^T and input gradient dX = dY.W).
 //
-// Work decomposition.  One workgroup (8 waves) owns a BM-token x 8-block-column tile of the result
-// (block columns of the *result*: block rows of W for the forward, block columns of W for dX).
-// Wave w serves token slice w & 3 (TM*32 tokens) and block-column half w >> 2 (4 block columns):
-// the two waves of a token slice sit on the same SIMD, so each SIMD sees every block product of
-// the tile and the four SIMDs stay balanced however uneven the pattern is, while one wave's LDS
-// and scalar work overlaps the other's matrix-core work.
+// Work decomposition.  One workgroup owns a BM-token x 8-block-column tile of the result (block
+// columns of the *result*: block rows of W for the forward, block columns of W for dX).  Its 8
+// compute waves are 4 token slices (TM*32 tokens each) x 2 block-column halves (4 block columns
+// each): the two waves of a token slice sit on the same SIMD, so each SIMD sees every block
+// product of the tile and the four SIMDs stay balanced however uneven the pattern is, while one
+// wave's LDS and scalar work overlaps the other's matrix-core work.
 //
 // Schedule.  What a tile has to do depends only on the pattern, so it is computed once per pattern
-// by dds_plan_kernel and kept in global memory (the "plan"): per group of 8 block columns the
-// merged list of k-blocks that any of them touches, with the present-column mask of each and the
-// data blocks in (k-block, column) order.  The matmul kernel reads it with scalar loads.
-//
-// Producer waves.  Issuing a DMA instruction blocks the issuing wave until the texture addresser
-// has taken it (about 25 cycles per instruction per CU when all waves stream), so waves that also
-// compute would add the copy time to their compute time.  With NP > 0 the workgroup has NP extra
-// waves that only issue DMA and wait for it; the 8 compute waves never touch global memory in the
-// main loop.  (fp32 spends 16x longer in the matrix cores per byte and keeps NP = 0.)
+// by dds_plan_kernel and kept in global memory (the "plan"): per group of 8 block columns one
+// 64-byte record per k-block that any of them touches (k-block, present-column mask, running entry
+// count, the data block of each column).  A workgroup copies its group's records to LDS once.
 //
 // Data movement.  A step covers SK k-blocks.  Its BM x 32 dense operand panels and its packed
 // blocks are copied global -> LDS by the DMA path (global_load_lds_dwordx4, no registers): panels
-// into a ring of RS step buffers, blocks into a ring of RB block slots, so that RS-1 steps of
-// loads are in flight while one is consumed.  Each wave waits for its own DMA instructions with an
-// exact s_waitcnt vmcnt(n); one barrier per step publishes the step to all waves.
+// into a ring of RS step buffers, blocks into a ring of RB block slots (entry e uses slot e % RB),
+// so that RS-1 steps of loads are in flight while one is consumed.  A wave waits for its own DMA
+// instructions with an exact s_waitcnt vmcnt(n); one barrier per step publishes the step.
+//
+// Copy waves.  Issuing a DMA instruction blocks the issuing wave until the texture addresser has
+// taken it (about 25 cycles per instruction per CU when all waves stream), so waves that also
+// compute would add the copy time to their compute time.  With NP > 0 the workgroup has NP extra
+// waves that only issue DMA and wait for it, and the compute waves never touch global memory in
+// the main loop.  (fp32 spends 16x longer in the matrix cores per byte and keeps NP = 0.)
 //
 // LDS layouts (16-byte chunks; a DMA instruction fills 64 consecutive chunks, lane p -> chunk p,
 // and each lane may fetch any global address, so the layout is chosen by the addresses):
@@ -33,32 +33,35 @@
 //   packed blocks for the forward stay as stored, [k][n]: bf16 operands are gathered k-major by
 //   ds_read_b64_tr_b16, fp32 operands are read one word per k.
 #pragma once
+#include <type_traits>
+
 #include "pbs_common.h"
 
 namespace pbs {
 
 constexpr int DDS_NB = 8;    // block columns per workgroup tile
-constexpr int DDS_NBW = 4;   // block columns per wave
-constexpr int DDS_NW = 8;    // waves per workgroup: 4 token slices x 2 column halves
+constexpr int DDS_NBW = 4;   // block columns per compute wave
+constexpr int DDS_NW = 8;    // compute waves per workgroup: 4 token slices x 2 column halves
 
-// ---- plan layout, in ints, per group of DDS_NB block columns (KB = K/32 k-blocks) ----
-//   [0..3]                 header: nk (present k-blocks), ne (entries), 0, 0
-//   [4 .. 4+4*(KB+1))      records, 4 ints each: k-block, present-column mask, entries before it, 0;
-//                          record nk is a sentinel holding ne in its third int
-//   [4+4*(KB+1) .. +8*KB)  data block of each entry, entries in (k-block, column) order
-static inline size_t dds_plan_group_ints(int KB) { return 4 + 4 * ((size_t)KB + 1) + (size_t)DDS_NB * KB; }
+// ---- plan layout per group of DDS_NB block columns: (KB + 2) records of 16 ints (KB = K/32) ----
+//   record 0        header: [0] = nk (present k-blocks), [1] = ne (entries)
+//   record 1 + i    i-th present k-block: [0..7] data block of each column or -1,
+//                   [8] k-block, [9] present-column mask, [10] entries before it
+//   record 1 + nk   sentinel: [10] = ne
+constexpr int DDS_REC_INTS = 16;
+constexpr int DDS_F_KB = 8, DDS_F_MASK = 9, DDS_F_CUM = 10;
+static inline size_t dds_plan_group_ints(int KB) { return ((size_t)KB + 2) * DDS_REC_INTS; }
 
 // One workgroup per group of 8 block columns merges their sorted block lists.
 __global__ __launch_bounds__(256) void dds_plan_kernel(const int32_t* __restrict__ ptr, const int32_t* __restrict__ idx,
                                                        int nblk_n, int KB, int nnz, int* plan, int group_ints) {
-    constexpr int NB = DDS_NB, SEG = 128, NT = 256;
+    constexpr int NB = DDS_NB, SEG = 128, NT = 256, R = DDS_REC_INTS;
     __shared__ int s_tbl[SEG * NB];
     __shared__ int s_ptr[NB + 1];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int nb0 = blockIdx.x * NB;
     int* out = plan + (size_t)blockIdx.x * group_ints;
-    int* rec = out + 4;
-    int* ent = out + 4 + 4 * (KB + 1);
+    int* rec = out + R;
     if (tid <= NB) {
         const int nb = nb0 + tid;
         s_ptr[tid] = ptr[nb < nblk_n ? nb : nblk_n];
@@ -96,17 +99,14 @@ __global__ __launch_bounds__(256) void dds_plan_kernel(const int32_t* __restrict
                 }
                 const int total = __shfl(incl, 63, 64);
                 if (cnt) {
-                    const int pos = nk + __popcll(m & ((1ull << lane) - 1ull));
-                    int e = ne + incl - cnt;
-                    rec[4 * pos + 0] = seg0 + kbl;
-                    rec[4 * pos + 1] = present;
-                    rec[4 * pos + 2] = e;
-                    rec[4 * pos + 3] = 0;
+                    int* r = rec + (size_t)(nk + __popcll(m & ((1ull << lane) - 1ull))) * R;
 #pragma unroll
-                    for (int j = 0; j < NB; ++j) {
-                        const int b = s_tbl[kbl * NB + j];
-                        if (b >= 0) ent[e++] = b;
-                    }
+                    for (int j = 0; j < NB; ++j) r[j] = s_tbl[kbl * NB + j];
+                    r[DDS_F_KB] = seg0 + kbl;
+                    r[DDS_F_MASK] = present;
+                    r[DDS_F_CUM] = ne + incl - cnt;
+#pragma unroll
+                    for (int j = DDS_F_CUM + 1; j < R; ++j) r[j] = 0;
                 }
                 nk += __popcll(m);
                 ne += total;
@@ -114,15 +114,10 @@ __global__ __launch_bounds__(256) void dds_plan_kernel(const int32_t* __restrict
         }
         __syncthreads();
     }
-    if (tid == 0) {
-        out[0] = nk;
-        out[1] = ne;
-        out[2] = 0;
-        out[3] = 0;
-        rec[4 * nk + 0] = 0;
-        rec[4 * nk + 1] = 0;
-        rec[4 * nk + 2] = ne;
-        rec[4 * nk + 3] = 0;
+    if (wave == 0 && lane < R) {
+        out[lane] = lane == 0 ? nk : (lane == 1 ? ne : 0);
+        int* r = rec + (size_t)nk * R;   // sentinel
+        r[lane] = lane < NB ? -1 : (lane == DDS_F_CUM ? ne : 0);
     }
 }
 
@@ -158,21 +153,22 @@ struct DdsCfg {
     static constexpr int PANEL_BYTES = BM * ROWB;        // one k-block of the dense operand
     static constexpr int PANEL_INSTR = PANEL_BYTES / 1024;
     static constexpr int A_PER_WAVE = PANEL_INSTR / ND;  // DMA instructions per issuing wave per k-block
+    static constexpr int COLS_PER_COPIER = DDS_NB / ND;  // block columns whose blocks a copy wave fetches
     static constexpr int STEP_BYTES = SK * PANEL_BYTES;
     static constexpr int BLK_BYTES = 1024 * E::ESZ;
     static constexpr int BLK_INSTR = BLK_BYTES / 1024;   // DMA instructions per packed block (2 or 4)
     static constexpr int A_RING_BYTES = RS * STEP_BYTES;
     static constexpr int B_RING_BYTES = RB * BLK_BYTES;
     static constexpr int RING_BYTES = A_RING_BYTES + B_RING_BYTES;
-    // the epilogue stages one 32-row x 128-column sub-tile per wave through LDS
+    // the epilogue stages one 32-row x 128-column sub-tile per compute wave through LDS
     static constexpr int EPI_WAVE_BYTES = 32 * 128 * E::ESZ;
     static constexpr int EPI_BYTES = NW * EPI_WAVE_BYTES;
-    static constexpr int LDS_BYTES = RING_BYTES > EPI_BYTES ? RING_BYTES : EPI_BYTES;
+    static constexpr int WORK_BYTES = RING_BYTES > EPI_BYTES ? RING_BYTES : EPI_BYTES;   // + the plan records
     static_assert(PANEL_INSTR % ND == 0 && A_PER_WAVE >= 1, "panel DMA must divide evenly over the issuing waves");
-    static_assert((ND & (ND - 1)) == 0, "issuing waves: power of two");
+    static_assert(DDS_NB % ND == 0 && COLS_PER_COPIER >= 1, "block columns must divide evenly over the issuing waves");
     static_assert(RS >= 2, "need at least two step buffers");
     static_assert(RB >= SK * DDS_NB && (RB & (RB - 1)) == 0, "the block ring holds one full step; power of two");
-    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+    static_assert(WORK_BYTES % 16 == 0, "alignment of the plan records");
 };
 
 // chunk swizzle of a row: bf16 rows have 4 chunks, fp32 rows 8
@@ -211,46 +207,205 @@ static __device__ __forceinline__ void wait_dma_and_barrier(int n) {
     }
 #undef PBS_W
 }
-static __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+// barrier of a wave that has no DMA in flight or does not care (its LDS accesses complete first)
+static __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+static __device__ __forceinline__ void drain_barrier() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 template <typename T, int TRANS, int TM, int SK, int RS, int RB, int NP>
 __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
     using C = DdsCfg<T, TRANS, TM, SK, RS, RB, NP>;
     using E = typename C::E;
-    constexpr int NB = DDS_NB, NBW = DDS_NBW, NW = DDS_NW, ND = C::ND, NQ = E::NQ, CPR = C::CPR;
+    constexpr int NB = DDS_NB, NBW = DDS_NBW, NW = DDS_NW, ND = C::ND, NQ = E::NQ, CPR = C::CPR, R = DDS_REC_INTS;
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
     unsigned char* const a_ring = smem;
     unsigned char* const b_ring = smem + C::A_RING_BYTES;
+    int* const s_plan = reinterpret_cast<int*>(smem + C::WORK_BYTES);   // this group's records
     const unsigned lds_a = (unsigned)(uintptr_t)a_ring;
     const unsigned lds_b = (unsigned)(uintptr_t)b_ring;
 
     const int tile = xcd_tile_id(blockIdx.x, g.m_tiles * g.n_groups);
     if (tile < 0) return;
-    const int mt = tile / g.n_groups;
-    const int ng = tile % g.n_groups;
+    // Order of the tiles inside an XCD's range: blocks of 4 token tiles x 8 column groups, so that the
+    // 32 workgroups an XCD runs at a time share 4 operand panels and 8 groups of weight blocks in
+    // its L2 (token-tile-major order would stream all the weights through every XCD's L2).
+    int mt, ng;
+    if ((g.n_groups % 8) == 0 && (g.m_tiles % 4) == 0) {
+        const int blk = tile >> 5, within = tile & 31;
+        const int ngb = blk % (g.n_groups / 8), mtb = blk / (g.n_groups / 8);
+        mt = mtb * 4 + (within >> 3);
+        ng = ngb * 8 + (within & 7);
+    } else {
+        mt = tile / g.n_groups;
+        ng = tile % g.n_groups;
+    }
     const int m0 = mt * C::BM;
     const int nb0 = ng * NB;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int ms = wave & 3;       // token slice
-    const int half = (wave >> 2) & 1;    // block-column half
-    const bool computes = wave < NW;
-    const bool copies = NP ? wave >= NW : true;
-    const int dw = NP ? (wave - NW) & (ND - 1) : wave;   // index among the waves that issue DMA
-    const int lrow = lane & 31;
-    const int h = lane >> 5;
 
-    const int* __restrict__ gp = g.plan + (size_t)ng * g.group_ints;
-    const int4* __restrict__ rec = reinterpret_cast<const int4*>(gp + 4);
-    const int* __restrict__ ent = gp + 4 + 4 * (g.K / 32 + 1);
-    const int nk = gp[0];
+    // ---- this group's plan records -> LDS ----
+    {
+        const int4* src = reinterpret_cast<const int4*>(g.plan + (size_t)ng * g.group_ints);
+        int4* dst = reinterpret_cast<int4*>(s_plan);
+        const int n4 = (2 + g.plan[(size_t)ng * g.group_ints]) * (R / 4);   // header + nk records + sentinel
+        for (int i = tid; i < n4; i += C::NT) dst[i] = src[i];
+    }
+    __syncthreads();
+    const int nk = __builtin_amdgcn_readfirstlane(s_plan[0]);
     const int ns = (nk + SK - 1) / SK;
+    // field f of present k-block i (i == nk: sentinel)
+    auto rec = [&](int i, int f) -> int { return __builtin_amdgcn_readfirstlane(s_plan[(1 + i) * R + f]); };
+    auto kend = [&](int s) -> int { const int i = (s + 1) * SK; return i < nk ? i : nk; };
+    auto cum = [&](int i) -> int { return rec(i, DDS_F_CUM); };
+
+    // Bookkeeping shared by all waves.  ce[d] = entries before the end of step s + d (read from the
+    // plan ahead of the barrier); step t may be issued while step s is the oldest unconsumed one if
+    // its panel buffer (t - s < RS) and its block slots (entries of steps s..t <= RB) are free.
+    struct Ends {
+        int c0, c1, c2, c3;   // scalars on purpose: an indexed array would go to scratch memory
+    };
+    static_assert(RS <= 4, "Ends holds four step ends");
+    auto load_ends = [&](Ends& ce, int s) {
+        ce.c0 = cum(kend(s));
+        ce.c1 = RS > 1 ? cum(kend(s + 1)) : 0;
+        ce.c2 = RS > 2 ? cum(kend(s + 2)) : 0;
+        ce.c3 = RS > 3 ? cum(kend(s + 3)) : 0;
+    };
+    auto can_issue = [&](int t, int s, int cum_s, const Ends& ce) -> bool {
+        const int d = t - s;
+        if (t >= ns || d >= RS) return false;
+        const int end = d == 0 ? ce.c0 : (d == 1 ? ce.c1 : (d == 2 ? ce.c2 : ce.c3));
+        return end - cum_s <= RB;
+    };
 
     const unsigned char* A_tile = static_cast<const unsigned char*>(g.a) + (size_t)m0 * g.K * E::ESZ;
     const unsigned char* D = static_cast<const unsigned char*>(g.data);
+
+    // =====================================================================================
+    // copy side: issue the DMA of step t; returns how many DMA instructions this wave issued
+    // =====================================================================================
+    struct Issuer {
+        unsigned a_voff[C::A_PER_WAVE];
+        unsigned b_voff[C::BLK_INSTR];
+    };
+    auto make_issuer = [&](int dw) -> Issuer {
+        // panel: copy wave dw fills instructions dw*A_PER_WAVE + i of every k-block; lane p of instruction
+        // q serves row q*RPI + p/CPR and physical chunk p%CPR, i.e. logical chunk (p%CPR) ^ swz(row)
+        Issuer is;
+#pragma unroll
+        for (int i = 0; i < C::A_PER_WAVE; ++i) {
+            const int q = dw * C::A_PER_WAVE + i;
+            const int row = q * C::RPI + lane / CPR;
+            const int chunk = (lane % CPR) ^ swz<CPR>(row);
+            int r = row;
+            if (m0 + r >= g.M) r = g.M - 1 - m0;   // rows past the end re-read the last row; never stored
+            is.a_voff[i] = (unsigned)r * (unsigned)(g.K * E::ESZ) + chunk * 16;
+        }
+        // packed block: instruction q of a block; forward keeps the block as stored, dX swizzles rows
+#pragma unroll
+        for (int q = 0; q < C::BLK_INSTR; ++q) {
+            if constexpr (TRANS) {
+                const int row = q * C::RPI + lane / CPR;
+                is.b_voff[q] = row * C::ROWB + ((lane % CPR) ^ swz<CPR>(row)) * 16;
+            } else {
+                is.b_voff[q] = q * 1024 + lane * 16;
+            }
+        }
+        return is;
+    };
+    auto issue_step = [&](const Issuer& is, int dw, int t) -> int {
+        const int i0 = t * SK, i1 = kend(t);
+        const unsigned stage = lds_a + (t % RS) * C::STEP_BYTES + dw * (C::A_PER_WAVE * 1024);
+        int n = 0;
+        for (int i = i0; i < i1; ++i) {
+            const unsigned char* src = uniform_ptr(A_tile + (size_t)rec(i, DDS_F_KB) * C::ROWB);
+            const unsigned dst = __builtin_amdgcn_readfirstlane(stage + (i - i0) * C::PANEL_BYTES);
+#pragma unroll
+            for (int q = 0; q < C::A_PER_WAVE; ++q) dma16(dst + q * 1024, src, is.a_voff[q]);
+            n += C::A_PER_WAVE;
+            // this wave fetches the blocks of columns dw, dw + ND, ...
+            const int mask = rec(i, DDS_F_MASK);
+            const int base = rec(i, DDS_F_CUM);
+#pragma unroll
+            for (int c = 0; c < C::COLS_PER_COPIER; ++c) {
+                const int j = dw + c * ND;
+                if ((mask >> j) & 1) {
+                    const int e = base + __popc(mask & ((1 << j) - 1));
+                    const unsigned char* bsrc = uniform_ptr(D + (size_t)rec(i, j) * C::BLK_BYTES);
+                    const unsigned bdst = __builtin_amdgcn_readfirstlane(lds_b + (e & (RB - 1)) * C::BLK_BYTES);
+#pragma unroll
+                    for (int q = 0; q < C::BLK_INSTR; ++q) dma16(bdst + q * 1024, bsrc, is.b_voff[q]);
+                    n += C::BLK_INSTR;
+                }
+            }
+        }
+        return n;
+    };
+
+    // the step loop of a wave that copies (and, with NP == 0, also computes through `compute`)
+    auto copy_loop = [&](int dw, auto&& compute) {
+        const Issuer is = make_issuer(dw);
+        int pend[RS];   // DMA counts of the issued, not yet consumed steps, oldest first
+#pragma unroll
+        for (int k = 0; k < RS; ++k) pend[k] = 0;
+        int npend = 0, next = 0, cum_s = 0;
+        auto push = [&](int c) {
+#pragma unroll
+            for (int k = 0; k < RS; ++k)
+                if (npend == k) pend[k] = c;
+            ++npend;
+        };
+        Ends ce;
+        load_ends(ce, 0);
+        while (can_issue(next, 0, 0, ce)) {
+            push(issue_step(is, dw, next));
+            ++next;
+        }
+        for (int s = 0; s < ns; ++s) {
+            if (next <= s) {
+                // the block ring could not take step s while step s-1 was in use
+                drain_barrier();
+                push(issue_step(is, dw, s));
+                next = s + 1;
+            }
+            load_ends(ce, s);
+            int later = 0;   // DMA of the steps after s may stay in flight
+#pragma unroll
+            for (int k = 1; k < RS; ++k) later += pend[k];
+            wait_dma_and_barrier(later);
+#pragma unroll
+            for (int k = 0; k + 1 < RS; ++k) pend[k] = pend[k + 1];
+            pend[RS - 1] = 0;
+            --npend;
+            // every wave is past step s-1 now: its buffers can be refilled
+            if (s > 0)
+                while (can_issue(next, s, cum_s, ce)) {
+                    push(issue_step(is, dw, next));
+                    ++next;
+                }
+            compute(s);
+            cum_s = ce.c0;
+        }
+        drain_barrier();   // the rings are reused by the epilogue
+    };
+
+    if constexpr (NP > 0) {
+        if (wave >= NW) {
+            copy_loop(wave - NW, [](int) {});
+            return;
+        }
+    }
+
+    // =====================================================================================
+    // compute side
+    // =====================================================================================
+    const int ms = wave & 3;            // token slice
+    const int half = (wave >> 2) & 1;   // block-column half
+    const int lrow = lane & 31;
+    const int h = lane >> 5;
 
     f32x16 acc[TM][NBW];
 #pragma unroll
@@ -260,38 +415,11 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    // ---- per-lane constants of the DMA address patterns ----
-    // panel: this wave fills instructions wave*A_PER_WAVE + i of every k-block; lane p of instruction q
-    // serves row q*RPI + p/CPR and physical chunk p%CPR, i.e. logical chunk (p%CPR) ^ swz(row)
-    unsigned a_voff[C::A_PER_WAVE];
-#pragma unroll
-    for (int i = 0; i < C::A_PER_WAVE; ++i) {
-        const int q = dw * C::A_PER_WAVE + i;
-        const int row = q * C::RPI + lane / CPR;
-        const int chunk = (lane % CPR) ^ swz<CPR>(row);
-        int r = row;
-        if (m0 + r >= g.M) r = g.M - 1 - m0;   // rows past the end re-read the last row; never stored
-        a_voff[i] = (unsigned)r * (unsigned)(g.K * E::ESZ) + chunk * 16;
-    }
-    // packed block: instruction q of a block; forward keeps the block as stored, dX swizzles rows
-    unsigned b_voff[C::BLK_INSTR];
-#pragma unroll
-    for (int q = 0; q < C::BLK_INSTR; ++q) {
-        if constexpr (TRANS) {
-            const int row = q * C::RPI + lane / CPR;
-            b_voff[q] = row * C::ROWB + ((lane % CPR) ^ swz<CPR>(row)) * 16;
-        } else {
-            b_voff[q] = q * 1024 + lane * 16;
-        }
-    }
     // per-lane offsets of the fragment reads
-    int a_frag_off[TM][NQ];
+    int a_frag_off[TM];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const int row = (ms * TM + i) * 32 + lrow;
-#pragma unroll
-        for (int q = 0; q < NQ; ++q) a_frag_off[i][q] = row * C::ROWB + (((h * NQ + q) ^ swz<CPR>(row)) * 16);
-    }
+    for (int i = 0; i < TM; ++i) a_frag_off[i] = ((ms * TM + i) * 32 + lrow) * C::ROWB;
+    const int a_sw = swz<CPR>(lrow);   // (ms*TM+i)*32 is a multiple of 32: the swizzle depends on lrow only
     int b_frag_off;
     if constexpr (TRANS) {
         b_frag_off = lrow * C::ROWB;   // + ((h*NQ+q) ^ swz(lrow)) * 16
@@ -303,44 +431,21 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
         const int l16 = lane & 15;
         b_frag_off = (16 * h + (l16 >> 2)) * 64 + (((lane >> 4) & 1) * 16 + (l16 & 3) * 4) * 2;
     }
-
-    auto kend = [&](int s) -> int { const int i = (s + 1) * SK; return i < nk ? i : nk; };
-    auto cum = [&](int i) -> int { return rec[i].z; };
-
-    // issue the DMA of step t; returns how many DMA instructions this wave issued
-    auto issue_step = [&](int t) -> int {
-        const int i0 = t * SK, i1 = kend(t);
-        const unsigned stage = lds_a + (t % RS) * C::STEP_BYTES + dw * (C::A_PER_WAVE * 1024);
-        for (int i = i0; i < i1; ++i) {
-            const unsigned char* src = uniform_ptr(A_tile + (size_t)rec[i].x * C::ROWB);
-            const unsigned dst = __builtin_amdgcn_readfirstlane(stage + (i - i0) * C::PANEL_BYTES);
+    int chunk_off[NQ];   // swizzled chunk offsets of this lane's k range, shared by panel rows and dX block rows
 #pragma unroll
-            for (int q = 0; q < C::A_PER_WAVE; ++q) dma16(dst + q * 1024, src, a_voff[q]);
-        }
-        const int e0 = cum(i0), e1 = cum(i1);
-        int n = (i1 - i0) * C::A_PER_WAVE;
-        for (int e = e0 + ((dw - e0) & (ND - 1)); e < e1; e += ND) {   // entries with e % ND == dw
-            const unsigned char* src = uniform_ptr(D + (size_t)ent[e] * C::BLK_BYTES);
-            const unsigned dst = __builtin_amdgcn_readfirstlane(lds_b + (e & (RB - 1)) * C::BLK_BYTES);
-#pragma unroll
-            for (int q = 0; q < C::BLK_INSTR; ++q) dma16(dst + q * 1024, src, b_voff[q]);
-            n += C::BLK_INSTR;
-        }
-        return n;
-    };
+    for (int q = 0; q < NQ; ++q) chunk_off[q] = ((h * NQ + q) ^ a_sw) * 16;
 
     auto load_a = [&](uint4 (&fa)[TM][NQ], const unsigned char* panel) {
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int q = 0; q < NQ; ++q) fa[i][q] = *reinterpret_cast<const uint4*>(panel + a_frag_off[i][q]);
+            for (int q = 0; q < NQ; ++q) fa[i][q] = *reinterpret_cast<const uint4*>(panel + a_frag_off[i] + chunk_off[q]);
     };
     auto load_b = [&](uint4 (&fb)[NQ], const unsigned char* pb) {
         if constexpr (TRANS) {
             const unsigned char* p = pb + b_frag_off;
-            const int sw = swz<CPR>(lrow);
 #pragma unroll
-            for (int q = 0; q < NQ; ++q) fb[q] = *reinterpret_cast<const uint4*>(p + (((h * NQ + q) ^ sw) * 16));
+            for (int q = 0; q < NQ; ++q) fb[q] = *reinterpret_cast<const uint4*>(p + chunk_off[q]);
         } else if constexpr (E::ESZ == 4) {
             const uint32_t* p = reinterpret_cast<const uint32_t*>(pb + b_frag_off);
 #pragma unroll
@@ -360,27 +465,32 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
             }
         }
     };
-    auto compute_step = [&](int s, const int4 (&recs)[SK]) {
-        const int i0 = s * SK;
+    // (mask, entries before) of the k-blocks of the current step, read ahead of the barrier
+    int st_mask[SK], st_cum[SK];
+    auto load_step_recs = [&](int s) {
+#pragma unroll
+        for (int k = 0; k < SK; ++k) {
+            const int i = s * SK + k;
+            st_mask[k] = i < nk ? rec(i, DDS_F_MASK) : 0;
+            st_cum[k] = rec(i < nk ? i : nk, DDS_F_CUM);
+        }
+    };
+    auto compute_step = [&](int s) {
         const unsigned char* stage = a_ring + (s % RS) * C::STEP_BYTES;
 #pragma unroll
         for (int k = 0; k < SK; ++k) {
-            const int4 r = recs[k];
-            const int mine = (i0 + k < nk) ? (r.y >> (NBW * half)) & ((1 << NBW) - 1) : 0;
+            const int mask = st_mask[k];
+            const int mine = (mask >> (NBW * half)) & ((1 << NBW) - 1);
             if (mine == 0) continue;
-            int e = r.z + (half ? __popc(r.y & ((1 << NBW) - 1)) : 0);
+            int e = st_cum[k] + (half ? __popc(mask & ((1 << NBW) - 1)) : 0);
             uint4 fa[TM][NQ];
-            uint4 fb[NQ];
-            // first block fragment and the panel fragments go out together: one LDS latency, not two
-            load_b(fb, b_ring + (e & (RB - 1)) * C::BLK_BYTES);
             load_a(fa, stage + k * C::PANEL_BYTES);
             // the accumulator index stays static; the branches are wave-uniform
-            bool first = true;
 #pragma unroll
             for (int j = 0; j < NBW; ++j) {
                 if ((mine >> j) & 1) {
-                    if (!first) load_b(fb, b_ring + (e & (RB - 1)) * C::BLK_BYTES);
-                    first = false;
+                    uint4 fb[NQ];
+                    load_b(fb, b_ring + (e & (RB - 1)) * C::BLK_BYTES);
                     ++e;
 #pragma unroll
                     for (int t = 0; t < TM; ++t) E::mma(acc[t][j], fa[t], fb);
@@ -390,73 +500,43 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
     };
 
 #ifdef PBS_EXP_TIMING
-    const bool prof_on = (tile == 300) && (lane == 0) && (wave == 0 || wave == NW + NP - 1);
-    const int prof_base = (wave == 0 ? 0 : 4096);
+    const bool prof_on = (tile == 300) && (lane == 0) && (wave == 0);
+    const int prof_base = 0;
     PBS_T(0);
 #endif
-    // ---- the steps ----
-    if (ns > 0) {
-        // DMA counts of the issued, not yet consumed steps, oldest first
-        int pend[RS];
-#pragma unroll
-        for (int k = 0; k < RS; ++k) pend[k] = 0;
-        int npend = 0;
-        int next = 0;
-        int cum_s = 0;   // entries before step s
-        auto can_issue = [&](int t, int s) -> bool {
-            return t < ns && t <= s + RS - 1 && cum(kend(t)) - cum_s <= RB;
-        };
-        auto push = [&](int c) {
-#pragma unroll
-            for (int k = 0; k < RS; ++k)
-                if (npend == k) pend[k] = c;
-            ++npend;
-        };
-        // every wave runs the same bookkeeping (the barriers must match); only the copying waves
-        // issue and wait for DMA, only the compute waves multiply
-        while (can_issue(next, 0)) {
-            push(copies ? issue_step(next) : 0);
-            ++next;
-        }
+    if constexpr (NP == 0) {
+        copy_loop(wave, [&](int s) {
+            load_step_recs(s);
+            compute_step(s);
+        });
+    } else {
+        // same bookkeeping as the copy waves (the barriers must match), without the DMA
+        int next = 0, cum_s = 0;
+        Ends ce;
+        load_ends(ce, 0);
+        while (can_issue(next, 0, 0, ce)) ++next;
         for (int s = 0; s < ns; ++s) {
             if (next <= s) {
-                // the block ring could not take step s while step s-1 was in use
                 lds_barrier();
-                push(copies ? issue_step(s) : 0);
                 next = s + 1;
             }
             PBS_T(8 + 4 * s + 0);
-            // records of this step: scalar loads, in flight across the wait
-            int4 recs[SK];
-#pragma unroll
-            for (int k = 0; k < SK; ++k) recs[k] = rec[s * SK + k < nk ? s * SK + k : nk];   // record nk is a sentinel
-            int later = 0;   // DMA of the steps after s may stay in flight
-#pragma unroll
-            for (int k = 1; k < RS; ++k) later += pend[k];
-            wait_dma_and_barrier(later);
+            load_ends(ce, s);
+            load_step_recs(s);
+            lds_barrier();
             PBS_T(8 + 4 * s + 1);
-#pragma unroll
-            for (int k = 0; k + 1 < RS; ++k) pend[k] = pend[k + 1];
-            pend[RS - 1] = 0;
-            --npend;
-            // every wave is past step s-1 now: its buffers can be refilled
             if (s > 0)
-                while (can_issue(next, s)) {
-                    push(copies ? issue_step(next) : 0);
-                    ++next;
-                }
+                while (can_issue(next, s, cum_s, ce)) ++next;
             PBS_T(8 + 4 * s + 2);
-            if (computes) compute_step(s, recs);
+            compute_step(s);
             PBS_T(8 + 4 * s + 3);
-            cum_s = cum(kend(s));
+            cum_s = ce.c0;
         }
+        PBS_T(1);
+        lds_barrier();
+        PBS_T(2);
     }
-    // the rings are reused by the epilogue: every wave must be done reading them
-    PBS_T(1);
-    lds_barrier();
-    PBS_T(2);
 
-    if (!computes) return;
     // ---- epilogue: each wave passes its 32 x 128 sub-tiles through its own LDS region so that the
     //      global stores are 16 bytes per lane along rows; bias fused ----
     T* out = static_cast<T*>(g.out);

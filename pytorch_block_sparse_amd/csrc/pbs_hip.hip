@@ -39,11 +39,15 @@ static int launch_dds(DdsArgs g, hipStream_t stream) {
     using C = DdsCfg<T, TRANS, TM, SK, RS, RB, NP>;
     static std::atomic<uint64_t> done{0};
     auto kernel = dds_kernel<T, TRANS, TM, SK, RS, RB, NP>;
-    if (int rc = raise_lds_limit(kernel, C::LDS_BYTES, done)) return rc;
+    constexpr int LDS_MAX = 160 * 1024;
+    // rings (or the epilogue staging) plus this group's plan records
+    const size_t lds = (size_t)C::WORK_BYTES + (size_t)g.group_ints * sizeof(int);
+    if (lds > (size_t)LDS_MAX) return PBS_ERR_TOO_LARGE;
+    if (int rc = raise_lds_limit(kernel, LDS_MAX, done)) return rc;
     g.m_tiles = (g.M + C::BM - 1) / C::BM;
     const long long tiles = (long long)g.m_tiles * g.n_groups;
     if (tiles > (1ll << 30)) return PBS_ERR_TOO_LARGE;
-    hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)tiles)), dim3(C::NT), C::LDS_BYTES, stream, g);
+    hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)tiles)), dim3(C::NT), lds, stream, g);
     return (int)hipGetLastError();
 }
 
