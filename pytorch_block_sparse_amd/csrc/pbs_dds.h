@@ -177,40 +177,6 @@ static __device__ __forceinline__ int swz(int r) {
     return CPR == 4 ? ((r >> 2) & 3) : ((r >> 1) & 7);
 }
 
-// a wave-uniform pointer, forced into scalar registers
-static __device__ __forceinline__ const unsigned char* uniform_ptr(const unsigned char* p) {
-    const uint64_t v = reinterpret_cast<uint64_t>(p);
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
-    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return reinterpret_cast<const unsigned char*>(((uint64_t)hi << 32) | lo);
-}
-
-// one DMA instruction: lane p copies the 16 bytes at base + voff to LDS chunk (lds_base/16 + p)
-static __device__ __forceinline__ void dma16(unsigned lds_base_uniform, const unsigned char* base_uniform, unsigned voff) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t"
-                 :
-                 : "s"(lds_base_uniform), "v"(voff), "s"(base_uniform)
-                 : "memory");
-}
-
-// wait until at most n (wave-uniform) of this wave's DMA loads are outstanding, make this wave's
-// LDS accesses complete, and meet the other waves.  Loads retire in order, so a smaller n than
-// necessary is only slower, never wrong.
-static __device__ __forceinline__ void wait_dma_and_barrier(int n) {
-#define PBS_W(N) case N: asm volatile("s_waitcnt vmcnt(" #N ") lgkmcnt(0)\n\ts_barrier" ::: "memory"); break;
-    switch (n) {
-        PBS_W(0) PBS_W(1) PBS_W(2) PBS_W(3) PBS_W(4) PBS_W(5) PBS_W(6) PBS_W(7) PBS_W(8)
-        PBS_W(9) PBS_W(10) PBS_W(11) PBS_W(12) PBS_W(13) PBS_W(14) PBS_W(15) PBS_W(16)
-        PBS_W(17) PBS_W(18) PBS_W(19) PBS_W(20) PBS_W(21) PBS_W(22) PBS_W(23) PBS_W(24)
-        PBS_W(25) PBS_W(26) PBS_W(27) PBS_W(28) PBS_W(29) PBS_W(30) PBS_W(31) PBS_W(32)
-        default: asm volatile("s_waitcnt vmcnt(32) lgkmcnt(0)\n\ts_barrier" ::: "memory"); break;
-    }
-#undef PBS_W
-}
-// barrier of a wave that has no DMA in flight or does not care (its LDS accesses complete first)
-static __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-static __device__ __forceinline__ void drain_barrier() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-
 template <typename T, int TRANS, int TM, int SK, int RS, int RB, int NP>
 __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
     using C = DdsCfg<T, TRANS, TM, SK, RS, RB, NP>;

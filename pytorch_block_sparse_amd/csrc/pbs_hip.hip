@@ -9,6 +9,7 @@
 #include "pbs_dds.h"
 #include "pbs_index.h"
 #include "pbs_sdd.h"
+#include "pbs_sdd_bf16.h"
 
 namespace pbs {
 
@@ -70,32 +71,27 @@ static int dispatch_dds(const DdsArgs& g, hipStream_t stream) {
 }
 
 // ---- sparse-output product ----
-template <typename T>
-struct SddShape;
-template <>
-struct SddShape<float> {
-    static constexpr int SR = 8, SC = 8, QW = 8, NW = 4;
+// fp32: 8 x 8 rectangles, 16-token chunks staged through registers; bf16: 16 x 16 rectangles,
+// 32-token chunks by DMA.
+struct SddShapeF32 {
+    static constexpr int SR = 8, SC = 8, QW = 8, NW = 4, TC = 16;
 };
-template <>
-struct SddShape<bf16_t> {
-    static constexpr int SR = 8, SC = 16, QW = 8, NW = 8;
+struct SddShapeBf16 {
+    static constexpr int SR = 16, SC = 16, QW = 10, TC = 32;
 };
 
 struct SddPlan {
     int tiles_r, tiles_c, nsplit, tokens_per_split;
 };
 
-template <typename T>
-static SddPlan plan_sdd(long long M, int N, int K) {
-    using S = SddShape<T>;
-    using C = SddCfg<T, S::SR, S::SC, S::QW, S::NW>;
+static SddPlan plan_sdd(long long M, int N, int K, int SR, int SC, int TC) {
     SddPlan p;
-    p.tiles_r = (N / 32 + S::SR - 1) / S::SR;
-    p.tiles_c = (K / 32 + S::SC - 1) / S::SC;
+    p.tiles_r = (N / 32 + SR - 1) / SR;
+    p.tiles_c = (K / 32 + SC - 1) / SC;
     const long long tiles = (long long)p.tiles_r * p.tiles_c;
-    const long long chunks = (M + C::TC - 1) / C::TC;
-    // aim at two workgroups per CU, but keep at least 8 chunks of tokens per slice
-    long long want = (512 + tiles - 1) / tiles;
+    const long long chunks = (M + TC - 1) / TC;
+    // aim at one or two workgroups per CU, but keep at least 8 chunks of tokens per slice
+    long long want = (256 + tiles - 1) / tiles;
     long long cap = chunks / 8;
     if (cap < 1) cap = 1;
     if (want > cap) want = cap;
@@ -103,18 +99,17 @@ static SddPlan plan_sdd(long long M, int N, int K) {
     const long long chunks_per = (chunks + want - 1) / want;
     p.nsplit = (int)((chunks + chunks_per - 1) / chunks_per);
     if (p.nsplit < 1) p.nsplit = 1;
-    p.tokens_per_split = (int)(chunks_per * C::TC);
+    p.tokens_per_split = (int)(chunks_per * TC);
     return p;
+}
+static SddPlan plan_sdd_for(int dtype, long long M, int N, int K) {
+    if (dtype == PBS_DTYPE_F32) return plan_sdd(M, N, K, SddShapeF32::SR, SddShapeF32::SC, SddShapeF32::TC);
+    return plan_sdd(M, N, K, SddShapeBf16::SR, SddShapeBf16::SC, SddShapeBf16::TC);
 }
 
 template <typename T>
-static int launch_sdd(SddArgs a, void* workspace, size_t workspace_bytes, hipStream_t stream) {
-    using S = SddShape<T>;
-    using C = SddCfg<T, S::SR, S::SC, S::QW, S::NW>;
-    static std::atomic<uint64_t> done{0};
-    auto kernel = sdd_kernel<T, S::SR, S::SC, S::QW, S::NW>;
-    if (int rc = raise_lds_limit(kernel, C::LDS_BYTES, done)) return rc;
-    const SddPlan p = plan_sdd<T>(a.M, a.N, a.K);
+static int launch_sdd(SddArgs a, int dtype, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    const SddPlan p = plan_sdd_for(dtype, a.M, a.N, a.K);
     a.tiles_r = p.tiles_r;
     a.tiles_c = p.tiles_c;
     a.nsplit = p.nsplit;
@@ -128,7 +123,23 @@ static int launch_sdd(SddArgs a, void* workspace, size_t workspace_bytes, hipStr
     }
     const long long wgs = (long long)p.tiles_r * p.tiles_c * p.nsplit;
     if (wgs > (1ll << 30)) return PBS_ERR_TOO_LARGE;
-    hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)wgs)), dim3(C::NT), C::LDS_BYTES, stream, a);
+    if constexpr (sizeof(T) == 4) {
+        using S = SddShapeF32;
+        using C = SddCfg<T, S::SR, S::SC, S::QW, S::NW>;
+        static_assert(C::TC == S::TC, "plan and kernel must agree on the chunk size");
+        static std::atomic<uint64_t> done{0};
+        auto kernel = sdd_kernel<T, S::SR, S::SC, S::QW, S::NW>;
+        if (int rc = raise_lds_limit(kernel, C::LDS_BYTES, done)) return rc;
+        hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)wgs)), dim3(C::NT), C::LDS_BYTES, stream, a);
+    } else {
+        using S = SddShapeBf16;
+        using C = SddBf16Cfg<S::QW>;
+        static_assert(C::TC == S::TC && C::SR == S::SR && C::SC == S::SC, "plan and kernel must agree");
+        static std::atomic<uint64_t> done{0};
+        auto kernel = sdd_bf16_kernel<S::QW>;
+        if (int rc = raise_lds_limit(kernel, C::LDS_BYTES, done)) return rc;
+        hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)wgs)), dim3(C::NT), C::LDS_BYTES, stream, a);
+    }
     int rc = (int)hipGetLastError();
     if (rc) return rc;
     if (p.nsplit > 1) {
@@ -233,10 +244,8 @@ size_t pbs_blocksparse_matmul_back_workspace_bytes(int64_t tokens, int out_featu
                                                    int dtype) {
     if (tokens <= 0 || out_features <= 0 || in_features <= 0 || nnz <= 0) return 0;
     if ((out_features % 32) || (in_features % 32)) return 0;
-    SddPlan p;
-    if (dtype == PBS_DTYPE_F32) p = plan_sdd<float>(tokens, out_features, in_features);
-    else if (dtype == PBS_DTYPE_BF16) p = plan_sdd<bf16_t>(tokens, out_features, in_features);
-    else return 0;
+    if (dtype != PBS_DTYPE_F32 && dtype != PBS_DTYPE_BF16) return 0;
+    const SddPlan p = plan_sdd_for(dtype, tokens, out_features, in_features);
     if (p.nsplit <= 1) return 0;
     return (size_t)nnz * 1024 * sizeof(float) * p.nsplit;
 }
@@ -273,8 +282,8 @@ int pbs_blocksparse_matmul_back(const void* dense_a, const void* dense_b, const 
     a.K = in_features;
     a.nnz = nnz;
     a.tiles_r = a.tiles_c = a.nsplit = a.tokens_per_split = 0;
-    if (dtype == PBS_DTYPE_F32) return launch_sdd<float>(a, workspace, workspace_bytes, s);
-    return launch_sdd<bf16_t>(a, workspace, workspace_bytes, s);
+    if (dtype == PBS_DTYPE_F32) return launch_sdd<float>(a, dtype, workspace, workspace_bytes, s);
+    return launch_sdd<bf16_t>(a, dtype, workspace, workspace_bytes, s);
 }
 
 }  // extern "C"
