@@ -1,0 +1,102 @@
+"""The C-ABI library: loads, exports every symbol the header declares, rejects bad arguments.
+
+No compute call is made here (no GPU): every call below returns from the argument checks,
+before the library touches the HIP runtime.
+"""
+import ctypes
+import os
+import re
+
+import pytest
+
+from pytorch_block_sparse_amd import native
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "pbs_hip.h")
+
+OK, ERR_NULL, ERR_SHAPE, ERR_DTYPE, ERR_ALIGN, ERR_WS, ERR_LARGE = 0, -1, -2, -3, -4, -5, -6
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(native.LIB_PATH):
+        pytest.skip("libpbs_hip.so is not built")
+    return native.load()
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(pbs_\w+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported(lib):
+    declared = _declared_symbols()
+    assert len(declared) >= 8
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in pbs_hip.h but not exported"
+    assert set(declared) == set(native.EXPORTED_SYMBOLS)
+
+
+def test_version_and_error_strings(lib):
+    text = open(HEADER).read()
+    assert lib.pbs_abi_version() == int(re.search(r"#define PBS_ABI_VERSION (\d+)", text).group(1))
+    assert native.error_string(0) == "ok"
+    for code in (ERR_NULL, ERR_SHAPE, ERR_DTYPE, ERR_ALIGN, ERR_WS, ERR_LARGE):
+        assert native.error_string(code).startswith("pbs:")
+    for name, code in re.findall(r"#define (PBS_ERR_\w+) \((-\d+)\)", text):
+        assert native.error_string(int(code)) != "pbs: unknown error code", name
+
+
+def test_matmul_argument_checks(lib):
+    p = ctypes.c_void_p(0x1000)  # never dereferenced: the checks fail first
+    null = ctypes.c_void_p(0)
+    f = lib.pbs_blocksparse_matmul
+    assert f(p, p, p, null, p, 4, 64, 64, 1, 1, 7, null) == ERR_DTYPE
+    assert f(p, p, p, null, p, 4, 65, 64, 1, 1, 0, null) == ERR_SHAPE
+    assert f(p, p, p, null, p, 4, 64, 33, 1, 1, 0, null) == ERR_SHAPE
+    assert f(p, p, p, null, p, -1, 64, 64, 1, 1, 0, null) == ERR_SHAPE
+    assert f(p, p, p, null, p, 4, 64, 64, 5, 1, 0, null) == ERR_LARGE      # more blocks than positions
+    assert f(p, p, p, null, p, 0, 64, 64, 1, 1, 0, null) == OK             # no tokens: nothing to do
+    assert f(null, p, p, null, p, 4, 64, 64, 1, 1, 0, null) == ERR_NULL
+    assert f(p, p, null, null, p, 4, 64, 64, 1, 1, 0, null) == ERR_NULL    # the plan is required
+    assert f(ctypes.c_void_p(0x1004), p, p, null, p, 4, 64, 64, 1, 1, 1, null) == ERR_ALIGN
+
+
+def test_plan_argument_checks(lib):
+    p = ctypes.c_void_p(0x1000)
+    null = ctypes.c_void_p(0)
+    nbytes = lib.pbs_blocksparse_matmul_plan_bytes(4096, 4096)
+    assert nbytes == 16 * (128 + 2) * 16 * 4   # 16 groups of 8 block columns, 64-byte records
+    assert lib.pbs_blocksparse_matmul_plan_bytes(100, 64) == 0
+    f = lib.pbs_blocksparse_matmul_plan
+    assert f(p, p, 64, 100, 1, p, 1 << 20, null) == ERR_SHAPE
+    assert f(null, p, 64, 64, 1, p, 1 << 20, null) == ERR_NULL
+    assert f(p, p, 64, 64, 1, p, 16, null) == ERR_WS
+
+
+def test_back_argument_checks(lib):
+    p = ctypes.c_void_p(0x1000)
+    null = ctypes.c_void_p(0)
+    f = lib.pbs_blocksparse_matmul_back
+    assert f(p, p, p, p, p, 8, 64, 64, 1, 9, null, 0, null) == ERR_DTYPE
+    assert f(p, p, p, p, p, 8, 64, 60, 1, 0, null, 0, null) == ERR_SHAPE
+    assert f(p, p, p, p, p, 8, 64, 64, 0, 0, null, 0, null) == OK           # no blocks: nothing to do
+    assert f(p, p, null, p, p, 8, 64, 64, 1, 0, null, 0, null) == ERR_NULL
+    assert f(ctypes.c_void_p(0x1008), p, p, p, p, 8, 64, 64, 1, 0, null, 0, null) == ERR_ALIGN
+    ws = lib.pbs_blocksparse_matmul_back_workspace_bytes
+    assert ws(0, 64, 64, 1, 0) == 0 and ws(16384, 4096, 4096, 4096, 5) == 0
+    need = ws(16384, 4096, 4096, 4096, 1)
+    assert need > 0 and need % (4096 * 1024 * 4) == 0
+    # the token range is split but no workspace is given
+    assert f(p, p, p, p, p, 16384, 4096, 4096, 4096, 1, null, 0, null) == ERR_WS
+
+
+def test_build_indices_argument_checks(lib):
+    p = ctypes.c_void_p(0x1000)
+    null = ctypes.c_void_p(0)
+    f = lib.pbs_build_indices
+    assert f(p, null, 0, 4, 0, p, p, p, p, p, p, null) == ERR_SHAPE
+    assert f(p, null, 4, 4, 17, p, p, p, p, p, p, null) == ERR_SHAPE
+    assert f(null, null, 4, 4, 2, p, p, p, p, p, p, null) == ERR_NULL
+    assert f(p, null, 4, 4, 2, null, p, p, p, p, p, null) == ERR_NULL
