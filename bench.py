@@ -21,6 +21,19 @@ sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}  # MI355X dense matrix peaks
 
+# HBM bytes per launch (fetch + write) of each kernel, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of this script, scaled by what the same counters read for a plain 256 MiB device
+# copy (fetch x2.0, write x1.0).  Counters cannot be read from inside the process, so the figures
+# are recorded here per workload and token count; other workloads report null.
+MIB = float(1 << 20)
+MEASURED_TRAFFIC = {
+    ("c4_4096x4096_d0.25_bf16", 16384): {
+        "fwd": (386.2 + 128.0) * MIB,
+        "dx": (386.1 + 128.0) * MIB,
+        "dw": (418.6 + 64.0 + 64.0 + 8.0) * MIB,   # partial sums, then the reduction
+    },
+}
+
 
 def parse():
     p = argparse.ArgumentParser()
@@ -32,6 +45,8 @@ def parse():
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     p.add_argument("--no-dense", action="store_true", help="skip the dense hipBLASLt leg")
     p.add_argument("--cpu-sample-tokens", type=int, default=2048)
+    p.add_argument("--copy-calibration", action="store_true",
+                   help="also run a plain 256 MiB device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     return p.parse_args()
 
 
@@ -140,7 +155,9 @@ def main():
     value = n_gemms * flops_gemm / (ms_step * 1e-3) / 1e12
     dom = max(per_kernel, key=per_kernel.get)
     achieved = flops_gemm / (per_kernel[dom] * 1e-3) / 1e12
-    kernel_names = {"fwd": "dds_kernel<TRANS=0>", "dx": "dds_kernel<TRANS=1>", "dw": "sdd_kernel(+sdd_reduce_kernel)"}
+    sdd = "sdd_bf16_kernel" if dname == "bf16" else "sdd_kernel"
+    kernel_names = {"fwd": "dds_kernel<TRANS=0>", "dx": "dds_kernel<TRANS=1>", "dw": sdd + " (+ sdd_reduce_kernel)"}
+    traffic = MEASURED_TRAFFIC.get((w.name, tokens), {}).get(dom)
 
     out = {
         "metric": "effective TFLOP/s fwd+bwd at 4096^2 d=0.25; % of MFMA peak; vs dense GEMM",
@@ -175,7 +192,9 @@ def main():
             "peak": PEAK_TFLOPS[dname],
             "unit": "TFLOP/s",
             "frac": achieved / PEAK_TFLOPS[dname],
-            "traffic": None,
+            "traffic": traffic,
+            "traffic_unit": "bytes per launch",
+            "flops_per_launch": flops_gemm,
         },
     }
 
@@ -200,6 +219,14 @@ def main():
             "speedup_sparse_vs_dense": ms_dense / ms_step,
         }
         del wd
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        out["copy_calibration_bytes"] = 1 << 28
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(w, min(args.cpu_sample_tokens, tokens))
