@@ -28,3 +28,12 @@ def assert_close(got, ref, dtype, what=""):
 
 def to64(t):
     return t.detach().to("cpu", torch.float64).numpy()
+
+
+def load_golden():
+    """The index-array vectors the reference's own tests hold (tests/golden/reference_index_vectors.json)."""
+    import json
+    import os
+
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_index_vectors.json")) as f:
+        return json.load(f)

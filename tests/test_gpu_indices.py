@@ -5,6 +5,7 @@ import torch
 
 from oracle import block_sparse_oracle as O
 from pytorch_block_sparse_amd import BlockSparseMatrix, native
+from tests.helpers import load_golden
 
 pytestmark = pytest.mark.gpu
 NAMES = ["blocks", "cols_a", "row_start_ends_a", "rows_b", "col_start_ends_b"]
@@ -19,18 +20,18 @@ def _device_indices(mask, block_ptr, cuda):
 
 def test_golden_vectors(cuda):
     """reference tests/test_basic.py:13-25 and tests/test_replace.py:23-43, on the device."""
-    m = BlockSparseMatrix.randn((128, 64), None, blocks=[(0, 0), (1, 0), (2, 0), (0, 1)], device=cuda, positive=True)
+    g = load_golden()
+    b, r = g["build"], g["replace"]
+    m = BlockSparseMatrix.randn(tuple(b["size"]), None, blocks=[tuple(x) for x in b["blocks_row_col"]], device=cuda,
+                                positive=True)
     assert m.cols_a.is_cuda and m.cols_a.dtype == torch.int32
-    assert m.row_start_ends_a.tolist() == [0, 2, 3, 4, 4]
-    assert m.cols_a.tolist() == [[0, 0], [1, 1], [0, 2], [0, 3]]
-    assert m.col_start_ends_b.tolist() == [0, 3, 4]
-    assert m.rows_b.tolist() == [[0, 0], [1, 2], [2, 3], [0, 1]]
-    assert m.blocks.tolist() == [0, 0, 1, 0, 0, 1, 0, 2]
+    for name in ("row_start_ends_a", "cols_a", "col_start_ends_b", "rows_b", "blocks"):
+        assert getattr(m, name).tolist() == b[name], name
     m.check_ = True
-    m.block_replace(torch.tensor([(3, 1, 0), (2, 1, 2), (1, 1, 1)]))
-    assert m.row_start_ends_a.tolist() == [0, 0, 1, 3, 4]
-    assert m.cols_a.tolist() == [[1, 1], [0, 3], [1, 2], [1, 0]]
-    assert m.block_mask_build(None).long().tolist() == [[0, 0], [0, 1], [1, 1], [0, 1]]
+    m.block_replace(torch.tensor(r["replacements"]))
+    assert m.row_start_ends_a.tolist() == r["row_start_ends_a"]
+    assert m.cols_a.tolist() == r["cols_a"]
+    assert m.block_mask_build(None).long().tolist() == r["block_mask"]
     m.check_with_dense(m.to_dense())
 
 

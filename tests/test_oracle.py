@@ -11,23 +11,15 @@ import numpy as np
 import pytest
 
 from oracle import block_sparse_oracle as O
+from tests.helpers import load_golden
 
-# ---- golden vectors held by the reference: tests/test_basic.py:13-25 -------------------------
-GOLD_SIZE = (128, 64)
-GOLD_BLOCKS = [(0, 0), (1, 0), (2, 0), (0, 1)]
-GOLD = dict(
-    row_start_ends_a=[0, 2, 3, 4, 4],
-    cols_a=[[0, 0], [1, 1], [0, 2], [0, 3]],
-    col_start_ends_b=[0, 3, 4],
-    rows_b=[[0, 0], [1, 2], [2, 3], [0, 1]],
-)
-# tests/test_replace.py:23-43
-GOLD_REPLACE = [(3, 1, 0), (2, 1, 2), (1, 1, 1)]
-GOLD_AFTER = dict(
-    row_start_ends_a=[0, 0, 1, 3, 4],
-    cols_a=[[1, 1], [0, 3], [1, 2], [1, 0]],
-    block_mask=[[0, 0], [0, 1], [1, 1], [0, 1]],
-)
+# ---- golden vectors held by the reference: tests/test_basic.py:13-25, tests/test_replace.py:23-43 ----
+_G = load_golden()
+GOLD_SIZE = tuple(_G["build"]["size"])
+GOLD_BLOCKS = [tuple(b) for b in _G["build"]["blocks_row_col"]]
+GOLD = {k: _G["build"][k] for k in ("row_start_ends_a", "cols_a", "col_start_ends_b", "rows_b")}
+GOLD_REPLACE = [tuple(r) for r in _G["replace"]["replacements"]]
+GOLD_AFTER = {k: _G["replace"][k] for k in ("row_start_ends_a", "cols_a", "block_mask")}
 
 
 def _gold_indices():
@@ -41,14 +33,14 @@ def test_build_indices_golden():
         assert idx[k].dtype == np.int32
         assert idx[k].tolist() == v, k
     # blocks: (col, row) of data block b; data blocks are in row-major order of the mask
-    assert idx["blocks"].tolist() == [0, 0, 1, 0, 0, 1, 0, 2]
+    assert idx["blocks"].tolist() == _G["build"]["blocks"]
 
 
 def test_block_info_golden():
     """tests/test_replace.py:29 block_info: position of every data block."""
     idx = _gold_indices()
     coo = O.build_coo_block_index(idx["row_start_ends_a"], idx["cols_a"])
-    assert coo.T.tolist() == [[0, 0], [0, 1], [1, 0], [2, 0]]
+    assert coo.T.tolist() == _G["build"]["block_info_row_col"]
 
 
 def test_block_replace_golden():
@@ -60,7 +52,7 @@ def test_block_replace_golden():
     assert after["cols_a"].tolist() == GOLD_AFTER["cols_a"]
     # data block b now sits where the replacement put it; block 3 stayed at (2, 0)
     coo = O.build_coo_block_index(after["row_start_ends_a"], after["cols_a"])
-    assert coo.T.tolist() == [[3, 1], [1, 1], [2, 1], [2, 0]]
+    assert coo.T.tolist() == _G["replace"]["block_info_row_col"]
 
 
 def test_block_replace_rejects_used_position():
