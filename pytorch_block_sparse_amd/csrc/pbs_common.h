@@ -122,7 +122,9 @@ static __device__ __forceinline__ void wait_dma_and_barrier(int n) {
         PBS_W(9) PBS_W(10) PBS_W(11) PBS_W(12) PBS_W(13) PBS_W(14) PBS_W(15) PBS_W(16)
         PBS_W(17) PBS_W(18) PBS_W(19) PBS_W(20) PBS_W(21) PBS_W(22) PBS_W(23) PBS_W(24)
         PBS_W(25) PBS_W(26) PBS_W(27) PBS_W(28) PBS_W(29) PBS_W(30) PBS_W(31) PBS_W(32)
-        default: asm volatile("s_waitcnt vmcnt(32) lgkmcnt(0)\n\ts_barrier" ::: "memory"); break;
+        PBS_W(33) PBS_W(34) PBS_W(35) PBS_W(36) PBS_W(37) PBS_W(38) PBS_W(39) PBS_W(40)
+        PBS_W(41) PBS_W(42) PBS_W(43) PBS_W(44) PBS_W(45) PBS_W(46) PBS_W(47) PBS_W(48)
+        default: asm volatile("s_waitcnt vmcnt(48) lgkmcnt(0)\n\ts_barrier" ::: "memory"); break;
     }
 #undef PBS_W
 }

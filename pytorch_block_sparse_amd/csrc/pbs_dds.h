@@ -222,23 +222,35 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
     __syncthreads();
     const int nk = __builtin_amdgcn_readfirstlane(s_plan[0]);
     const int ns = (nk + SK - 1) / SK;
-    // field f of present k-block i (i == nk: sentinel)
-    auto rec = [&](int i, int f) -> int { return __builtin_amdgcn_readfirstlane(s_plan[(1 + i) * R + f]); };
+    // Plan fields are read a whole step at a time: lane l of fetch_recs(t) holds int (l % 16) of the
+    // (l / 16)-th k-block record of step t (records past the last one read the sentinel), and single
+    // fields are then picked with v_readlane -- one LDS round trip per step instead of one per field.
     auto kend = [&](int s) -> int { const int i = (s + 1) * SK; return i < nk ? i : nk; };
-    auto cum = [&](int i) -> int { return rec(i, DDS_F_CUM); };
+    auto fetch_recs = [&](int t) -> int {
+        int i = t * SK + (lane >> 4);
+        if (i > nk) i = nk;
+        return s_plan[(1 + i) * R + (lane & 15)];
+    };
+    auto field = [&](int vrec, int k, int f) -> int { return __builtin_amdgcn_readlane(vrec, k * R + f); };
 
-    // Bookkeeping shared by all waves.  ce[d] = entries before the end of step s + d (read from the
-    // plan ahead of the barrier); step t may be issued while step s is the oldest unconsumed one if
-    // its panel buffer (t - s < RS) and its block slots (entries of steps s..t <= RB) are free.
+    // Bookkeeping shared by all waves.  ce.c<d> = entries before the end of step s + d; step t may be
+    // issued while step s is the oldest unconsumed one if its panel buffer (t - s < RS) and its block
+    // slots (entries of steps s..t <= RB) are free.
     struct Ends {
         int c0, c1, c2, c3;   // scalars on purpose: an indexed array would go to scratch memory
     };
     static_assert(RS <= 4, "Ends holds four step ends");
-    auto load_ends = [&](Ends& ce, int s) {
-        ce.c0 = cum(kend(s));
-        ce.c1 = RS > 1 ? cum(kend(s + 1)) : 0;
-        ce.c2 = RS > 2 ? cum(kend(s + 2)) : 0;
-        ce.c3 = RS > 3 ? cum(kend(s + 3)) : 0;
+    static_assert(SK * R <= 64, "one lane per record int of a step");
+    auto fetch_ends = [&](int s) -> int {   // lane d: entries before the end of step s + d
+        int i = (s + (lane & 3) + 1) * SK;
+        if (i > nk) i = nk;
+        return s_plan[(1 + i) * R + DDS_F_CUM];
+    };
+    auto unpack_ends = [&](Ends& ce, int v) {
+        ce.c0 = __builtin_amdgcn_readlane(v, 0);
+        ce.c1 = RS > 1 ? __builtin_amdgcn_readlane(v, 1) : 0;
+        ce.c2 = RS > 2 ? __builtin_amdgcn_readlane(v, 2) : 0;
+        ce.c3 = RS > 3 ? __builtin_amdgcn_readlane(v, 3) : 0;
     };
     auto can_issue = [&](int t, int s, int cum_s, const Ends& ce) -> bool {
         const int d = t - s;
@@ -247,6 +259,10 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
         return end - cum_s <= RB;
     };
 
+#ifdef PBS_EXP_TIMING
+    const bool prof_on = (tile == 300) && (lane == 0) && (wave == 0 || wave == NW);
+    const int prof_base = wave == 0 ? 0 : 4096;
+#endif
     const unsigned char* A_tile = static_cast<const unsigned char*>(g.a) + (size_t)m0 * g.K * E::ESZ;
     const unsigned char* D = static_cast<const unsigned char*>(g.data);
 
@@ -282,29 +298,33 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
         }
         return is;
     };
-    auto issue_step = [&](const Issuer& is, int dw, int t) -> int {
-        const int i0 = t * SK, i1 = kend(t);
+    auto issue_step = [&](const Issuer& is, int dw, int t, int vrec) -> int {
+        const int cnt = kend(t) - t * SK;   // k-blocks of this step
         const unsigned stage = lds_a + (t % RS) * C::STEP_BYTES + dw * (C::A_PER_WAVE * 1024);
         int n = 0;
-        for (int i = i0; i < i1; ++i) {
-            const unsigned char* src = uniform_ptr(A_tile + (size_t)rec(i, DDS_F_KB) * C::ROWB);
-            const unsigned dst = __builtin_amdgcn_readfirstlane(stage + (i - i0) * C::PANEL_BYTES);
 #pragma unroll
-            for (int q = 0; q < C::A_PER_WAVE; ++q) dma16(dst + q * 1024, src, is.a_voff[q]);
-            n += C::A_PER_WAVE;
-            // this wave fetches the blocks of columns dw, dw + ND, ...
-            const int mask = rec(i, DDS_F_MASK);
-            const int base = rec(i, DDS_F_CUM);
+        for (int k = 0; k < SK; ++k) {
+            if (k < cnt) {
+                const unsigned char* src = uniform_ptr(A_tile + (size_t)field(vrec, k, DDS_F_KB) * C::ROWB);
+                const unsigned dst = __builtin_amdgcn_readfirstlane(stage + k * C::PANEL_BYTES);
 #pragma unroll
-            for (int c = 0; c < C::COLS_PER_COPIER; ++c) {
-                const int j = dw + c * ND;
-                if ((mask >> j) & 1) {
-                    const int e = base + __popc(mask & ((1 << j) - 1));
-                    const unsigned char* bsrc = uniform_ptr(D + (size_t)rec(i, j) * C::BLK_BYTES);
-                    const unsigned bdst = __builtin_amdgcn_readfirstlane(lds_b + (e & (RB - 1)) * C::BLK_BYTES);
+                for (int q = 0; q < C::A_PER_WAVE; ++q) dma16(dst + q * 1024, src, is.a_voff[q]);
+                n += C::A_PER_WAVE;
+                // this wave fetches the blocks of columns dw, dw + ND, ...
+                const int mask = field(vrec, k, DDS_F_MASK);
+                const int base = field(vrec, k, DDS_F_CUM);
 #pragma unroll
-                    for (int q = 0; q < C::BLK_INSTR; ++q) dma16(bdst + q * 1024, bsrc, is.b_voff[q]);
-                    n += C::BLK_INSTR;
+                for (int c = 0; c < C::COLS_PER_COPIER; ++c) {
+                    const int j = dw + c * ND;
+                    if ((mask >> j) & 1) {
+                        const int e = base + __popc(mask & ((1 << j) - 1));
+                        const unsigned char* bsrc =
+                            uniform_ptr(D + (size_t)__builtin_amdgcn_readlane(vrec, k * R + j) * C::BLK_BYTES);
+                        const unsigned bdst = __builtin_amdgcn_readfirstlane(lds_b + (e & (RB - 1)) * C::BLK_BYTES);
+#pragma unroll
+                        for (int q = 0; q < C::BLK_INSTR; ++q) dma16(bdst + q * 1024, bsrc, is.b_voff[q]);
+                        n += C::BLK_INSTR;
+                    }
                 }
             }
         }
@@ -325,23 +345,29 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
             ++npend;
         };
         Ends ce;
-        load_ends(ce, 0);
+        unpack_ends(ce, fetch_ends(0));
+        int vrec = fetch_recs(0);   // records of step `next`, fetched one issue ahead
         while (can_issue(next, 0, 0, ce)) {
-            push(issue_step(is, dw, next));
+            push(issue_step(is, dw, next, vrec));
             ++next;
+            vrec = fetch_recs(next);
         }
         for (int s = 0; s < ns; ++s) {
             if (next <= s) {
                 // the block ring could not take step s while step s-1 was in use
                 drain_barrier();
-                push(issue_step(is, dw, s));
+                push(issue_step(is, dw, s, vrec));
                 next = s + 1;
+                vrec = fetch_recs(next);
             }
-            load_ends(ce, s);
+            PBS_T(8 + 4 * s + 0);
+            const int vends = fetch_ends(s);
             int later = 0;   // DMA of the steps after s may stay in flight
 #pragma unroll
             for (int k = 1; k < RS; ++k) later += pend[k];
             wait_dma_and_barrier(later);
+            PBS_T(8 + 4 * s + 1);
+            unpack_ends(ce, vends);
 #pragma unroll
             for (int k = 0; k + 1 < RS; ++k) pend[k] = pend[k + 1];
             pend[RS - 1] = 0;
@@ -349,10 +375,13 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
             // every wave is past step s-1 now: its buffers can be refilled
             if (s > 0)
                 while (can_issue(next, s, cum_s, ce)) {
-                    push(issue_step(is, dw, next));
+                    push(issue_step(is, dw, next, vrec));
                     ++next;
+                    vrec = fetch_recs(next);
                 }
+            PBS_T(8 + 4 * s + 2);
             compute(s);
+            PBS_T(8 + 4 * s + 3);
             cum_s = ce.c0;
         }
         drain_barrier();   // the rings are reused by the epilogue
@@ -434,11 +463,11 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
     // (mask, entries before) of the k-blocks of the current step, read ahead of the barrier
     int st_mask[SK], st_cum[SK];
     auto load_step_recs = [&](int s) {
+        const int v = fetch_recs(s);
 #pragma unroll
         for (int k = 0; k < SK; ++k) {
-            const int i = s * SK + k;
-            st_mask[k] = i < nk ? rec(i, DDS_F_MASK) : 0;
-            st_cum[k] = rec(i < nk ? i : nk, DDS_F_CUM);
+            st_mask[k] = s * SK + k < nk ? field(v, k, DDS_F_MASK) : 0;
+            st_cum[k] = field(v, k, DDS_F_CUM);
         }
     };
     auto compute_step = [&](int s) {
@@ -465,11 +494,7 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
         }
     };
 
-#ifdef PBS_EXP_TIMING
-    const bool prof_on = (tile == 300) && (lane == 0) && (wave == 0);
-    const int prof_base = 0;
     PBS_T(0);
-#endif
     if constexpr (NP == 0) {
         copy_loop(wave, [&](int s) {
             load_step_recs(s);
@@ -479,7 +504,7 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
         // same bookkeeping as the copy waves (the barriers must match), without the DMA
         int next = 0, cum_s = 0;
         Ends ce;
-        load_ends(ce, 0);
+        unpack_ends(ce, fetch_ends(0));
         while (can_issue(next, 0, 0, ce)) ++next;
         for (int s = 0; s < ns; ++s) {
             if (next <= s) {
@@ -487,9 +512,10 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
                 next = s + 1;
             }
             PBS_T(8 + 4 * s + 0);
-            load_ends(ce, s);
+            const int vends = fetch_ends(s);
             load_step_recs(s);
             lds_barrier();
+            unpack_ends(ce, vends);
             PBS_T(8 + 4 * s + 1);
             if (s > 0)
                 while (can_issue(next, s, cum_s, ce)) ++next;

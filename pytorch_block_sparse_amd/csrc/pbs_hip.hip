@@ -7,6 +7,7 @@
 
 #include "pbs_common.h"
 #include "pbs_dds.h"
+#include "pbs_dds16.h"
 #include "pbs_index.h"
 #include "pbs_sdd.h"
 #include "pbs_sdd_bf16.h"
@@ -52,6 +53,62 @@ static int launch_dds(DdsArgs g, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
+// ---- wide-tile persistent bf16 kernel ----
+// The plan buffer holds the narrow plan first, then (when k is a multiple of 64) the wide one.
+static inline size_t narrow_plan_bytes(int n, int k) {
+    const size_t groups = ((size_t)(n / 32) + DDS_NB - 1) / DDS_NB;
+    return groups * dds_plan_group_ints(k / 32) * sizeof(int);
+}
+static inline size_t wide_plan_bytes(int n, int k) {
+    if (k % 64) return 0;
+    const size_t groups = ((size_t)(n / 32) + D16_NB - 1) / D16_NB;
+    return groups * dds16_plan_group_ints(k / 32) * sizeof(int);
+}
+
+constexpr int D16_RS = 3, D16_RB = 32, D16_NP = 4;
+
+// Whether the wide kernel serves this problem: k-pairs need k % 64 == 0, the plan records of a group
+// must fit in LDS beside the rings, and there must be enough tiles to give every CU one.
+static bool wide_kernel_fits(long long M, int n, int k) {
+    using C = D16Cfg<D16_RS, D16_RB, D16_NP>;
+    if (k % 64) return false;
+    const size_t lds = (size_t)C::WORK_BYTES + dds16_plan_group_ints(k / 32) * sizeof(int);
+    if (lds > 160 * 1024) return false;
+    const long long tiles = ((M + C::BM - 1) / C::BM) * ((n / 32 + D16_NB - 1) / D16_NB);
+    return tiles >= 256;
+}
+
+template <int TRANS>
+static int launch_dds16(const DdsArgs& g, hipStream_t stream) {
+    using C = D16Cfg<D16_RS, D16_RB, D16_NP>;
+    static std::atomic<uint64_t> done{0};
+    auto kernel = dds16_kernel<TRANS, D16_RS, D16_RB, D16_NP>;
+    D16Args a;
+    a.a = g.a;
+    a.data = g.data;
+    a.plan = reinterpret_cast<const int*>(reinterpret_cast<const unsigned char*>(g.plan) + narrow_plan_bytes(g.N, g.K));
+    a.bias = g.bias;
+    a.out = g.out;
+    a.M = g.M;
+    a.N = g.N;
+    a.K = g.K;
+    a.nnz = g.nnz;
+    a.m_tiles = (g.M + C::BM - 1) / C::BM;
+    a.n_groups = (g.N / 32 + D16_NB - 1) / D16_NB;
+    a.group_ints = (int)dds16_plan_group_ints(g.K / 32);
+    // about one workgroup per CU, each walking the token tiles p, p + P, ... of its column group
+    int P = 256 / a.n_groups;
+    if (P < 1) P = 1;
+    if (P > a.m_tiles) P = a.m_tiles;
+    a.wg_per_group = P;
+    const size_t lds = (size_t)C::WORK_BYTES + (size_t)a.group_ints * sizeof(int);
+    if (int rc = raise_lds_limit(kernel, 160 * 1024, done)) return rc;
+    const long long grid = 8ll * a.n_groups * ((P + 7) / 8);
+    if (grid > (1ll << 30)) return PBS_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(C::NT), lds, stream, a);
+    return (int)hipGetLastError();
+}
+
 // Tile shapes: 256 tokens x 8 block columns when that still gives every CU a tile, else 128 tokens.
 // bf16 steps cover two k-blocks (the matrix cores go through a k-block 16x faster than in fp32).
 template <typename T, int TRANS>
@@ -64,6 +121,7 @@ static int dispatch_dds(const DdsArgs& g, hipStream_t stream) {
 #ifdef PBS_EXP_BF16_CFG
         return launch_dds<T, TRANS, PBS_EXP_BF16_CFG>(g, stream);
 #else
+        if (wide_kernel_fits(g.M, g.N, g.K)) return launch_dds16<TRANS>(g, stream);
         if (big_tiles >= 256) return launch_dds<T, TRANS, 2, 2, 3, 16, 4>(g, stream);
         return launch_dds<T, TRANS, 1, 2, 3, 16, 4>(g, stream);
 #endif
@@ -195,8 +253,7 @@ int pbs_build_indices(const uint8_t* mask, const int64_t* block_ptr, int X, int 
 
 size_t pbs_blocksparse_matmul_plan_bytes(int n, int k) {
     if (n <= 0 || k <= 0 || (n % 32) || (k % 32)) return 0;
-    const size_t groups = ((size_t)(n / 32) + DDS_NB - 1) / DDS_NB;
-    return groups * dds_plan_group_ints(k / 32) * sizeof(int);
+    return narrow_plan_bytes(n, k) + wide_plan_bytes(n, k);
 }
 
 int pbs_blocksparse_matmul_plan(const int32_t* ptr, const int32_t* indices, int n, int k, int nnz, void* plan,
@@ -208,6 +265,13 @@ int pbs_blocksparse_matmul_plan(const int32_t* ptr, const int32_t* indices, int 
     const int groups = (n / 32 + DDS_NB - 1) / DDS_NB;
     hipLaunchKernelGGL(dds_plan_kernel, dim3(groups), dim3(256), 0, static_cast<hipStream_t>(stream), ptr, indices, n / 32,
                        k / 32, nnz, static_cast<int*>(plan), (int)dds_plan_group_ints(k / 32));
+    if (int rc = (int)hipGetLastError()) return rc;
+    if (wide_plan_bytes(n, k)) {
+        const int groups16 = (n / 32 + D16_NB - 1) / D16_NB;
+        int* wide = reinterpret_cast<int*>(static_cast<unsigned char*>(plan) + narrow_plan_bytes(n, k));
+        hipLaunchKernelGGL(dds16_plan_kernel, dim3(groups16), dim3(256), 0, static_cast<hipStream_t>(stream), ptr, indices,
+                           n / 32, k / 32, nnz, wide, (int)dds16_plan_group_ints(k / 32));
+    }
     return (int)hipGetLastError();
 }
 

@@ -164,3 +164,58 @@ def test_benchmark_config_bf16_full_size_properties(cuda):
     assert err < 3 * 2.0 ** -8 * ref.abs().max().item(), err
     y_small = m.reverse_matmul(xd[1024:1536], True)
     assert torch.equal(y_small, y[1024:1536])
+
+
+# Shapes that the wide-tile persistent bf16 kernel serves (at least 256 tiles of 128 tokens x 512
+# result columns, contraction size a multiple of 64): one k-pair per tile, token tail, a last column
+# group with a single block column, full density (every step fills the block ring), persistence over
+# several token tiles.
+@pytest.mark.parametrize("in_f,out_f,tokens,density", [
+    (64, 512, 32768 + 5, 0.5),
+    (128, 1056, 11011, 1.0),
+    (512, 2048, 8192 + 77, 0.3),
+    (320, 512, 33000, 0.07),
+])
+def test_wide_tile_kernel_shapes(cuda, in_f, out_f, tokens, density):
+    print(f"wide {in_f}->{out_f} d={density} tokens={tokens}", flush=True)
+    n_blocks = max(1, int(density * (in_f // 32) * (out_f // 32)))
+    m = _matrix(out_f, in_f, None, n_blocks, torch.bfloat16, cuda, seed=21)
+    _check_all(m, (tokens,), torch.bfloat16, cuda, 23, f"wide {in_f}->{out_f} d={density}")
+
+
+def test_wide_tile_kernel_empty_group_and_bias(cuda):
+    """Blocks only in the first 8 block rows of W: the second group of 16 result columns has no block."""
+    in_f, out_f, tokens = 256, 1024, 16384 + 130
+    rng = np.random.RandomState(5)
+    blocks = sorted({(int(r), int(c)) for r, c in zip(rng.randint(0, 8, 40), rng.randint(0, 8, 40))})
+    m = _matrix(out_f, in_f, blocks, None, torch.bfloat16, cuda, seed=9)
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn((tokens, in_f), generator=g).to(torch.bfloat16)
+    bias = torch.randn((out_f,), generator=g).to(torch.bfloat16)
+    coo = m.build_coo_block_index().cpu().numpy()
+    w_dense = O.to_dense(to64(m.data), coo, (out_f, in_f))
+    y_ref = to64(x) @ w_dense.T
+    xd = x.to(cuda)
+    y = m.reverse_matmul(xd, True)
+    assert (y[:, 256:] == 0).all()
+    assert_close(y, y_ref, torch.bfloat16, "empty group fwd")
+    yb = m.reverse_matmul(xd, True, bias=bias.to(cuda))
+    assert_close(yb, y_ref + to64(bias)[None, :], torch.bfloat16, "empty group fwd + bias")
+    assert torch.equal(yb[:, 256:], bias.to(cuda)[None, 256:].expand(tokens, -1))
+
+
+def test_benchmark_config_bf16_4096_tokens(cuda):
+    """4096 -> 4096, density 0.25, bf16 at 4096 tokens: the smallest token count of this layer that runs
+    the wide-tile kernel in both directions; oracle-checked in full."""
+    w = workloads.WORKLOADS["c4_4096x4096_d0.25_bf16"]
+    blocks, data, x, dy = workloads.make_inputs(w, tokens=4096)
+    m = BlockSparseMatrix.zeros((w.out_features, w.in_features), blocks=blocks, device="cpu", dtype=w.dtype)
+    with torch.no_grad():
+        m.data.copy_(data)
+    coo = m.build_coo_block_index().numpy()
+    y_ref, dx_ref, dw_ref = O.linear_fwd_bwd(to64(x), to64(dy), to64(data), coo, tuple(m.shape))
+    m = m.to(cuda)
+    xd, dyd = x.to(cuda), dy.to(cuda)
+    assert_close(m.reverse_matmul(xd, True), y_ref, w.dtype, "c4/4096 fwd")
+    assert_close(m.reverse_matmul(dyd, False), dx_ref, w.dtype, "c4/4096 dx")
+    assert_close(m.matmul_with_output_sparse_support(dyd, xd), dw_ref, w.dtype, "c4/4096 dw")
