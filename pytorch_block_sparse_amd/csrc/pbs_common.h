@@ -128,6 +128,28 @@ static __device__ __forceinline__ void wait_dma_and_barrier(int n) {
     }
 #undef PBS_W
 }
+// the 4-byte form: lane p copies the 4 bytes at base + voff to LDS word (lds_base/4 + p)
+static __device__ __forceinline__ void dma4(unsigned lds_base_uniform, const unsigned char* base_uniform, unsigned voff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2\n\t"
+                 :
+                 : "s"(lds_base_uniform), "v"(voff), "s"(base_uniform)
+                 : "memory");
+}
+
+// wait until at most n (wave-uniform) of this wave's DMA loads are outstanding
+static __device__ __forceinline__ void wait_dma(int n) {
+#define PBS_W(N) case N: asm volatile("s_waitcnt vmcnt(" #N ")" ::: "memory"); break;
+    switch (n) {
+        PBS_W(0) PBS_W(1) PBS_W(2) PBS_W(3) PBS_W(4) PBS_W(5) PBS_W(6) PBS_W(7) PBS_W(8)
+        PBS_W(9) PBS_W(10) PBS_W(11) PBS_W(12) PBS_W(13) PBS_W(14) PBS_W(15) PBS_W(16)
+        PBS_W(17) PBS_W(18) PBS_W(19) PBS_W(20) PBS_W(21) PBS_W(22) PBS_W(23) PBS_W(24)
+        PBS_W(25) PBS_W(26) PBS_W(27) PBS_W(28) PBS_W(29) PBS_W(30) PBS_W(31) PBS_W(32)
+        PBS_W(33) PBS_W(34) PBS_W(35) PBS_W(36) PBS_W(37) PBS_W(38) PBS_W(39) PBS_W(40)
+        PBS_W(41) PBS_W(42) PBS_W(43) PBS_W(44) PBS_W(45) PBS_W(46) PBS_W(47) PBS_W(48)
+        default: asm volatile("s_waitcnt vmcnt(48)" ::: "memory"); break;
+    }
+#undef PBS_W
+}
 // barrier of a wave that has no DMA in flight or does not care (its LDS accesses complete first)
 static __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 static __device__ __forceinline__ void drain_barrier() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); }

@@ -9,19 +9,32 @@
 // about 1.5x faster than 64-byte pieces.
 //
 // Persistent workgroups.  A workgroup keeps one group of 16 block columns (its plan records stay in
-// LDS) and walks several token tiles.  The 4 copy waves issue the DMA of the following steps across
-// tile boundaries while the 8 compute waves are still in the epilogue of the previous tile, so the
-// first-load latency of a tile and the store burst of its epilogue overlap with useful work.
+// LDS) and walks several token tiles; the stream of steps simply continues across tile boundaries.
+//
+// No barriers in the step loop.  With a barrier per step all waves of a SIMD do their bookkeeping at
+// the same time and their matrix work at the same time, so the matrix cores idle during the former,
+// and every step lasts as long as its slowest wave (the pattern gives the waves different numbers of
+// blocks).  Instead the 4 copy waves and the 8 compute waves run as producers and consumers of the
+// two rings and publish their progress in LDS words:
+//   landed[c]   steps whose DMA from copy wave c has arrived, modulo 256.  The copy wave does not wait
+//               for its loads: after the loads of step t it issues one more DMA that copies the number
+//               (t + 1) % 256 from a table in global memory onto landed[c]; a wave's loads complete in
+//               order, so the number appears when the step's operands are in place;
+//   done[w]     (steps, block entries) compute wave w has finished reading.
+// A compute wave starts step u when every landed[c] has reached u + 1; a copy wave issues step t when every
+// done[w].steps >= t - RS + 1 (panel buffer free) and entries_end(t) - min done[w].entries <= RB
+// (block slots free).  All counters only grow, each has one writer, and waves poll with s_sleep, so
+// waves drift apart by up to the ring depth and one wave's overhead overlaps another's matrix work.
 //
 // Plan (built by dds16_plan_kernel per pattern and direction): per group of 16 block columns, one
 // 256-byte record per k-pair that any of them touches:
-//   [0..15]  data block of each column in the even k-block of the pair, or -1
-//   [16..31] the same for the odd k-block
+//   [0..31]  data blocks of the pair's entries, in entry order (unused places hold -1)
 //   [32] k-pair index   [33] presence mask (bit 16*odd + column)   [34] entries before this pair
 // preceded by a header record ([0] = pairs present, [1] = entries) and followed by a sentinel
-// ([34] = entries).  Entries are numbered in mask-bit order; entry e lives in block slot e % RB.
+// ([34] = entries).  The entries of a pair are its present (k-block, column) positions in mask-bit
+// order: even k-block first, columns ascending.  Entry e lives in block slot e % RB.
 //
-// LDS: [A ring: RS steps x 16 KB][block ring: RB x 2 KB][epilogue staging: 8 x 2304 B][plan records].
+// LDS: [A ring: RS steps x 16 KB][block ring: RB x 2 KB][epilogue staging: 8 x 2304 B][progress words][plan records].
 // Panel rows are 128 bytes (8 chunks of 16 bytes); chunk c of row r sits at position c ^ ((r >> 1) & 7),
 // which makes the 16-byte fragment reads of 16 consecutive rows conflict-free.  Packed blocks are laid
 // out as in the narrow kernel (pbs_dds.h).
@@ -36,10 +49,11 @@ constexpr int D16_REC = 64;     // ints per plan record
 constexpr int D16_F_PAIR = 32, D16_F_MASK = 33, D16_F_CUM = 34;
 constexpr int D16_BM = 128;     // tokens per tile
 static inline size_t dds16_plan_group_ints(int KB) { return ((size_t)(KB / 2) + 2) * D16_REC; }
+constexpr int D16_SEQ_INTS = 256;   // table 0..255 behind the plan records: source of the progress DMA
 
 // One workgroup per group of 16 block columns merges their sorted block lists into k-pair records.
 __global__ __launch_bounds__(256) void dds16_plan_kernel(const int32_t* __restrict__ ptr, const int32_t* __restrict__ idx,
-                                                         int nblk_n, int KB, int nnz, int* plan, int group_ints) {
+                                                         int nblk_n, int KB, int nnz, int* plan, int group_ints, int* seq) {
     constexpr int NB = D16_NB, SEG = 128, NT = 256, R = D16_REC;
     __shared__ int s_tbl[SEG * NB];
     __shared__ int s_ptr[NB + 1];
@@ -84,8 +98,13 @@ __global__ __launch_bounds__(256) void dds16_plan_kernel(const int32_t* __restri
             const int total = __shfl(incl, 63, 64);
             if (cnt) {
                 int* r = rec + (size_t)(np + __popcll(m & ((1ull << lane) - 1ull))) * R;
+                int n = 0;
 #pragma unroll
-                for (int j = 0; j < 2 * NB; ++j) r[j] = s_tbl[lane * 2 * NB + j];
+                for (int j = 0; j < 2 * NB; ++j) {
+                    const int b = s_tbl[lane * 2 * NB + j];
+                    if (b >= 0) r[n++] = b;
+                }
+                for (; n < 2 * NB; ++n) r[n] = -1;
                 r[D16_F_PAIR] = seg0 / 2 + lane;
                 r[D16_F_MASK] = (int)present;
                 r[D16_F_CUM] = ne + incl - cnt;
@@ -97,6 +116,7 @@ __global__ __launch_bounds__(256) void dds16_plan_kernel(const int32_t* __restri
         }
         __syncthreads();
     }
+    if (blockIdx.x == 0) seq[tid] = tid;   // the numbers the copy waves publish their progress with
     if (wave == 0) {
         out[lane] = lane == 0 ? np : (lane == 1 ? ne : 0);
         int* r = rec + (size_t)np * R;   // sentinel
@@ -108,6 +128,7 @@ struct D16Args {
     const void* a;         // [M, K] row-major bf16
     const void* data;      // [nnz*32, 32] bf16
     const int* plan;       // built by dds16_plan_kernel for this pattern and direction
+    const int* seq;        // the table 0..255 written by dds16_plan_kernel
     const void* bias;      // nullptr or [N]
     void* out;             // [M, N] row-major
     int M, N, K, nnz;
@@ -115,9 +136,12 @@ struct D16Args {
     int wg_per_group;      // workgroups that share the token tiles of one column group
 };
 
-template <int RS, int RB, int NP>
+template <int TM_, int RS, int RB, int NP>
 struct D16Cfg {
-    static constexpr int NW = 8, NT = (NW + NP) * 64, BM = D16_BM, TM = 2, NBW = 4;
+    // 8 compute waves = (4 / TM) token slices of TM * 32 tokens x (2 * TM) column groups of NBW = 8 / TM block
+    // columns; wave w has slice w % (4 / TM), so the waves that share a SIMD (w, w + 4) share their slice
+    static constexpr int NW = 8, NT = (NW + NP) * 64, BM = D16_BM, TM = TM_, NBW = 8 / TM_, NSL = 4 / TM_;
+    static_assert(TM_ == 1 || TM_ == 2, "token sub-slices per wave");
     static constexpr int ROWB = 128;                          // one panel row: 64 k values
     static constexpr int PANEL_BYTES = BM * ROWB;             // 16 KB per step
     static constexpr int A_PER_WAVE = PANEL_BYTES / 1024 / NP;
@@ -128,7 +152,13 @@ struct D16Cfg {
     static constexpr int STAGE_ROW = 136;                     // bf16 elements per staged row (128 + padding)
     static constexpr int STAGE_WAVE_BYTES = 2304;             // 8 rows x 272 B, rounded up
     static constexpr int STAGE_BYTES = NW * STAGE_WAVE_BYTES;
-    static constexpr int WORK_BYTES = A_RING_BYTES + B_RING_BYTES + STAGE_BYTES;   // + the plan records
+    // progress words: done steps [NW][64] then done entries [NW][64] (every lane of a compute wave writes
+    // its own copy, lane 0's is read), then landed [NP][64] (the progress DMA writes one copy per lane)
+    static constexpr int DONE_BYTES = NW * 64 * 8;
+    static constexpr int FLAG_BYTES = DONE_BYTES + NP * 256;   // landed[c]: 64 copies of one word per copy wave
+    static constexpr int FLAG_OFF = A_RING_BYTES + B_RING_BYTES + STAGE_BYTES;
+    static constexpr int WORK_BYTES = FLAG_OFF + FLAG_BYTES;   // + the plan records
+    static constexpr int SPIN_LIMIT = 1 << 20;                // polls before a wave gives up waiting
     static constexpr int MAX_STEP_DMA = A_PER_WAVE + 2 * COLS_PER_COPIER * 2;      // per copy wave
     static_assert(NP == 4, "four copy waves: one per SIMD");
     static_assert(RB >= 2 * D16_NB && (RB & (RB - 1)) == 0, "the block ring holds one full step; power of two");
@@ -137,9 +167,9 @@ struct D16Cfg {
     static_assert(WORK_BYTES % 256 == 0, "alignment of the plan records");
 };
 
-template <int TRANS, int RS, int RB, int NP>
+template <int TRANS, int TM_, int RS, int RB, int NP>
 __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
-    using C = D16Cfg<RS, RB, NP>;
+    using C = D16Cfg<TM_, RS, RB, NP>;
     using E = Elem<bf16_t>;
     constexpr int NBW = C::NBW, NW = C::NW, TM = C::TM, R = D16_REC;
 
@@ -164,12 +194,15 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
     const int ntiles = (g.m_tiles - p + g.wg_per_group - 1) / g.wg_per_group;   // token tiles p, p + P, ...
     const int nb0 = ng * D16_NB;
 
-    // ---- this group's plan records -> LDS ----
+    // ---- this group's plan records -> LDS; progress words start at zero ----
+    int* const s_done = reinterpret_cast<int*>(smem + C::FLAG_OFF);                     // [2][NW][64]
+    int* const s_landed = reinterpret_cast<int*>(smem + C::FLAG_OFF + C::DONE_BYTES);   // [NP]
     {
         const int4* src = reinterpret_cast<const int4*>(g.plan + (size_t)ng * g.group_ints);
         int4* dst = reinterpret_cast<int4*>(s_plan);
         const int n4 = (2 + g.plan[(size_t)ng * g.group_ints]) * (R / 4);   // header + records + sentinel
         for (int i = tid; i < n4; i += C::NT) dst[i] = src[i];
+        for (int i = tid; i < C::FLAG_BYTES / 4; i += C::NT) s_done[i] = 0;
     }
     __syncthreads();
     const int ns = __builtin_amdgcn_readfirstlane(s_plan[0]);   // steps (k-pairs) per tile
@@ -183,32 +216,6 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
 
     // lane l: int l of the record of step s of a tile
     auto fetch_rec = [&](int s) -> int { return s_plan[(1 + s) * R + lane]; };
-    // lane d (0..3): entries before the end of global step u + d, where u is step s of tile j
-    auto fetch_ends = [&](int j, int s) -> int {
-        int sd = s + (lane & 3), jd = j;
-        while (sd >= ns) {   // at most once unless a tile has fewer than 4 steps
-            sd -= ns;
-            ++jd;
-        }
-        return jd * ne + s_plan[(2 + sd) * R + D16_F_CUM];
-    };
-    struct Ends {
-        int c0, c1, c2, c3;
-    };
-    auto unpack_ends = [&](Ends& ce, int v) {
-        ce.c0 = __builtin_amdgcn_readlane(v, 0);
-        ce.c1 = __builtin_amdgcn_readlane(v, 1);
-        ce.c2 = RS > 2 ? __builtin_amdgcn_readlane(v, 2) : 0;
-        ce.c3 = RS > 3 ? __builtin_amdgcn_readlane(v, 3) : 0;
-    };
-    // global step t may be issued while u is the oldest unconsumed one (ent_u entries before it) if its
-    // panel buffer (t - u < RS) and its block slots (entries of steps u..t <= RB) are free
-    auto can_issue = [&](int t, int u, int ent_u, const Ends& ce) -> bool {
-        const int d = t - u;
-        if (t >= nsteps || d >= RS) return false;
-        const int end = d == 0 ? ce.c0 : (d == 1 ? ce.c1 : (d == 2 ? ce.c2 : ce.c3));
-        return end - ent_u <= RB;
-    };
 
     const unsigned char* A = static_cast<const unsigned char*>(g.a);
     const unsigned char* D = static_cast<const unsigned char*>(g.data);
@@ -240,112 +247,111 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
                 b_voff[q] = q * 1024 + lane * 16;
             }
         }
-        // issue the DMA of global step t = step s of tile j (records in vrec); returns the instruction count
-        auto issue_step = [&](int t, int j, int vrec) -> int {
+        // per token tile: global offsets of this wave's panel rows (rows past the end re-read the last
+        // row; they are never stored)
+        unsigned a_voff[C::A_PER_WAVE];
+        const unsigned char* a_tile = A;
+        auto enter_tile = [&](int j) {
             const int m0 = (p + j * g.wg_per_group) * C::BM;
-            const int last_row = g.M - 1 - m0;   // rows past the end re-read the last row; never stored
-            const int pair = __builtin_amdgcn_readlane(vrec, D16_F_PAIR);
-            const unsigned mask = (unsigned)__builtin_amdgcn_readlane(vrec, D16_F_MASK);
-            const int base = j * ne + __builtin_amdgcn_readlane(vrec, D16_F_CUM);
-            const unsigned char* src = uniform_ptr(A + (size_t)m0 * a_row_bytes + (size_t)pair * C::ROWB);
-            const unsigned stage =
-                __builtin_amdgcn_readfirstlane(lds_a + (t % RS) * C::PANEL_BYTES + dw * (C::A_PER_WAVE * 1024));
-            int n = 0;
-#ifndef PBS_EXP_NO_A
+            const int last_row = g.M - 1 - m0;
 #pragma unroll
             for (int q = 0; q < C::A_PER_WAVE; ++q) {
                 const int r = a_row[q] < last_row ? a_row[q] : last_row;
-                dma16(stage + q * 1024, src, (unsigned)r * (unsigned)a_row_bytes + a_chunk[q]);
+                a_voff[q] = (unsigned)r * (unsigned)a_row_bytes + a_chunk[q];
             }
+            a_tile = uniform_ptr(A + (size_t)m0 * a_row_bytes);
+        };
+        // Issue the DMA of global step t (panel buffer `stage`, records in vrec, e0 entries before it).
+        // The blocks of a step are dealt to the copy waves by entry number (dw, dw + 4, ...).
+        // Returns the instruction count.
+        auto issue_step = [&](unsigned stage, int vrec, int e0, int cnt) -> int {
+            int n = 0;
+#ifndef PBS_EXP_NO_A
+            const int pair = __builtin_amdgcn_readlane(vrec, D16_F_PAIR);
+            const unsigned char* src = uniform_ptr(a_tile + (size_t)pair * C::ROWB);
+#pragma unroll
+            for (int q = 0; q < C::A_PER_WAVE; ++q) dma16(stage + q * 1024, src, a_voff[q]);
             n = C::A_PER_WAVE;
 #endif
-            // this wave fetches the blocks of columns dw, dw + 4, dw + 8, dw + 12 of both k-blocks
+#ifndef PBS_EXP_NO_B
 #pragma unroll
-            for (int kk = 0; kk < 2; ++kk) {
-#pragma unroll
-                for (int c = 0; c < C::COLS_PER_COPIER; ++c) {
-                    const int bit = 16 * kk + dw + c * NP;
-#ifdef PBS_EXP_NO_B
-                    if (false) {
-#else
-                    if ((mask >> bit) & 1u) {
-#endif
-                        const int e = base + __popc(mask & ((1u << bit) - 1u));
-                        const unsigned char* bsrc =
-                            uniform_ptr(D + (size_t)__builtin_amdgcn_readlane(vrec, bit) * C::BLK_BYTES);
-                        const unsigned bdst = __builtin_amdgcn_readfirstlane(lds_b + (e & (RB - 1)) * C::BLK_BYTES);
-                        dma16(bdst, bsrc, b_voff[0]);
-                        dma16(bdst + 1024, bsrc, b_voff[1]);
-                        n += 2;
-                    }
+            for (int k = 0; k < 2 * D16_NB / NP; ++k) {
+                const int i = dw + k * NP;
+                if (i < cnt) {
+                    const unsigned id = (unsigned)__builtin_amdgcn_readlane(vrec, i);
+                    const unsigned char* bsrc = uniform_ptr(D + ((size_t)id << 11));
+                    const unsigned bdst = lds_b + (((unsigned)(e0 + i) & (RB - 1)) << 11);
+                    dma16(bdst, bsrc, b_voff[0]);
+                    dma16(bdst + 1024, bsrc, b_voff[1]);
+                    n += 2;
                 }
             }
+#endif
             return n;
         };
 
-        int pend[RS];   // DMA counts of the issued, not yet consumed steps, oldest first
-#pragma unroll
-        for (int k = 0; k < RS; ++k) pend[k] = 0;
-        int npend = 0;
-        auto push = [&](int c) {
-#pragma unroll
-            for (int k = 0; k < RS; ++k)
-                if (npend == k) pend[k] = c;
-            ++npend;
+        // minimum over the compute waves of (steps done, entries done): lanes 0..7 read lane 0's pair of
+        // each wave, three row shifts bring the minimum to lane 7
+        auto consumers_done = [&](int& steps, int& entries) {
+            const volatile int* pw = s_done + (lane & 7) * 64;
+            int a = pw[0], b = pw[NW * 64];
+#define PBS_MIN_SHR(SH)                                                                  \
+    {                                                                                    \
+        const int a2 = __builtin_amdgcn_update_dpp(a, a, 0x110 + SH, 0xf, 0xf, false);   \
+        const int b2 = __builtin_amdgcn_update_dpp(b, b, 0x110 + SH, 0xf, 0xf, false);   \
+        a = a2 < a ? a2 : a;                                                             \
+        b = b2 < b ? b2 : b;                                                             \
+    }
+            PBS_MIN_SHR(1) PBS_MIN_SHR(2) PBS_MIN_SHR(4)
+#undef PBS_MIN_SHR
+            steps = __builtin_amdgcn_readlane(a, 7);
+            entries = __builtin_amdgcn_readlane(b, 7);
         };
-        int next = 0, jn = 0, sn = 0;   // next global step to issue = step sn of tile jn
+        const unsigned landed_lds = (unsigned)(uintptr_t)(s_landed + dw * 64);
+        int jn = 0, sn = 0;          // step t is step sn of tile jn
         int vrec = fetch_rec(0);
-        auto issue_next = [&]() {
-            push(issue_step(next, jn, vrec));
-            ++next;
+        unsigned stage = lds_a + dw * (C::A_PER_WAVE * 1024);   // this wave's part of panel buffer t % RS
+        const unsigned stage_end = stage + RS * C::PANEL_BYTES;
+        enter_tile(0);
+        for (int t = 0; t < nsteps; ++t) {
+            PBS_T(8 + 4 * t + 0);
+            // wait until the panel buffer and the block slots of step t are free
+            const int cnt = __popc((unsigned)__builtin_amdgcn_readlane(vrec, D16_F_MASK));
+            const int e0 = jn * ne + __builtin_amdgcn_readlane(vrec, D16_F_CUM);
+            const int end_t = e0 + cnt;
+            for (int spin = 0; spin < C::SPIN_LIMIT; ++spin) {
+                int steps, entries;
+                consumers_done(steps, entries);
+                if (steps >= t - RS + 1 && end_t - entries <= RB) break;
+                __builtin_amdgcn_s_sleep(1);
+            }
+            wait_dma(63 - C::MAX_STEP_DMA - 1);   // the counter of outstanding loads has 6 bits
+            asm volatile("" ::: "memory");
+            PBS_T(8 + 4 * t + 1);
+            const int n_t = issue_step(stage, vrec, e0, cnt);
+            stage += C::PANEL_BYTES;
+            if (stage == stage_end) stage -= RS * C::PANEL_BYTES;
             if (++sn == ns) {
                 sn = 0;
                 ++jn;
+                if (t + 1 < nsteps) enter_tile(jn);
             }
-            vrec = fetch_rec(sn);   // consumed at the next issue: the LDS latency is hidden
-        };
-        Ends ce;
-        unpack_ends(ce, fetch_ends(0, 0));
-        int ent_u = 0;
-        while (can_issue(next, 0, 0, ce)) issue_next();
-        int j = 0, s = 0;
-        for (int u = 0; u < nsteps; ++u) {
-            if (next <= u) {
-                // the block ring could not take step u while step u-1 was in use
-                drain_barrier();
-                issue_next();
-            }
-            PBS_T(8 + 4 * u + 0);
-            const int vends = fetch_ends(j, s);
-            int later = 0;   // DMA of the steps after u may stay in flight
-#pragma unroll
-            for (int k = 1; k < RS; ++k) later += pend[k];
-            wait_dma_and_barrier(later);
-            PBS_T(8 + 4 * u + 1);
-            unpack_ends(ce, vends);
-#pragma unroll
-            for (int k = 0; k + 1 < RS; ++k) pend[k] = pend[k + 1];
-            pend[RS - 1] = 0;
-            --npend;
-            // every wave is past step u-1 now: its buffers can be refilled
-            if (u > 0)
-                while (can_issue(next, u, ent_u, ce)) issue_next();
-            PBS_T(8 + 4 * u + 2);
-            PBS_T(8 + 4 * u + 3);
-            ent_u = ce.c0;
-            if (++s == ns) {
-                s = 0;
-                ++j;
-            }
+            vrec = fetch_rec(sn);   // consumed in the next iteration: the LDS latency is hidden
+            PBS_T(8 + 4 * t + 2);
+            // behind the operands of step t: the number t + 1 (mod 256) onto this wave's landed words
+            dma4(landed_lds, uniform_ptr(reinterpret_cast<const unsigned char*>(g.seq + ((t + 1) & 255))), 0u);
+            (void)n_t;
+            PBS_T(8 + 4 * t + 3);
         }
+        wait_dma(0);
         return;
     }
 
     // =====================================================================================
     // compute waves
     // =====================================================================================
-    const int ms = wave & 1;        // token slice (64 tokens)
-    const int quarter = wave >> 1;  // 4 block columns
+    const int ms = wave % C::NSL;       // token slice (TM * 32 tokens)
+    const int quarter = wave / C::NSL;  // group of NBW block columns
     const int lrow = lane & 31;
     const int h = lane >> 5;
 
@@ -362,26 +368,20 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
         const int l16 = lane & 15;
         b_lane_off = (16 * h + (l16 >> 2)) * 64 + (((lane >> 4) & 1) * 16 + (l16 & 3) * 4) * 2;
     }
-    auto load_a = [&](uint4 (&fa)[TM][2], const unsigned char* panel, int kk) {
+    // fragments of one 16-byte register index q: 8 of the 16 k values a lane holds of a k-block
+    auto load_a = [&](uint4 (&fa)[TM], const unsigned char* panel, int kk, int q) {
+        const unsigned char* pq = panel + (a_lane_off ^ (kk * 64 + q * 16));
 #pragma unroll
-        for (int q = 0; q < 2; ++q) {
-            const unsigned char* pq = panel + (a_lane_off ^ (kk * 64 + q * 16));
-#pragma unroll
-            for (int i = 0; i < TM; ++i) fa[i][q] = *reinterpret_cast<const uint4*>(pq + i * 32 * C::ROWB);
-        }
+        for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const uint4*>(pq + i * 32 * C::ROWB);
     };
-    auto load_b = [&](uint4 (&fb)[2], const unsigned char* pb) {
+    auto load_b = [&](const unsigned char* pb, int q) -> uint4 {
         if constexpr (TRANS) {
-#pragma unroll
-            for (int q = 0; q < 2; ++q) fb[q] = *reinterpret_cast<const uint4*>(pb + (b_lane_off ^ (q * 16)));
+            return *reinterpret_cast<const uint4*>(pb + (b_lane_off ^ (q * 16)));
         } else {
             const unsigned char* pp = pb + b_lane_off;
-#pragma unroll
-            for (int q = 0; q < 2; ++q) {
-                const uint2 lo = tr16_b64(pp + (8 * q) * 64);
-                const uint2 hi = tr16_b64(pp + (8 * q + 4) * 64);
-                fb[q] = make_uint4(lo.x, lo.y, hi.x, hi.y);
-            }
+            const uint2 lo = tr16_b64(pp + (8 * q) * 64);
+            const uint2 hi = tr16_b64(pp + (8 * q + 4) * 64);
+            return make_uint4(lo.x, lo.y, hi.x, hi.y);
         }
     };
 
@@ -410,62 +410,72 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
         asm volatile("" : "+v"(l));
         const int er = l & 31, eh = l >> 5;
         const int m0 = (p + j * g.wg_per_group) * C::BM;
-        float bv[NBW];
-#pragma unroll
-        for (int jc = 0; jc < NBW; ++jc) {
-            const int col = col0 + jc * 32 + er;
-            bv[jc] = (bias && col < g.N) ? E::to_f32(bias[col]) : 0.f;
-        }
         bf16_t* st_w = stage + (4 * eh) * C::STAGE_ROW + er;                    // + vv rows, + jc*32
         const int rd_r = l >> 4, rd_c = (l & 15) * 8;
         const bf16_t* st_r = stage + rd_r * C::STAGE_ROW + rd_c;                // + 4 rows for the second read
-        const int col = col0 + rd_c;
 #pragma unroll
-        for (int t = 0; t < TM; ++t) {
+        for (int cg = 0; cg < NBW / 4; ++cg) {   // 4 block columns (128 result columns) at a time
+            float bv[4];
 #pragma unroll
-            for (int gq = 0; gq < 4; ++gq) {
+            for (int jc = 0; jc < 4; ++jc) {
+                const int col = col0 + (cg * 4 + jc) * 32 + er;
+                bv[jc] = (bias && col < g.N) ? E::to_f32(bias[col]) : 0.f;
+            }
+            const int col = col0 + cg * 128 + rd_c;
 #pragma unroll
-                for (int jc = 0; jc < NBW; ++jc)
+            for (int t = 0; t < TM; ++t) {
 #pragma unroll
-                    for (int vv = 0; vv < 4; ++vv)
-                        st_w[vv * C::STAGE_ROW + jc * 32] = E::from_f32(acc[t][jc][4 * gq + vv] + bv[jc]);
+                for (int gq = 0; gq < 4; ++gq) {
 #pragma unroll
-                for (int pp = 0; pp < 2; ++pp) {
-                    const uint4 val = *reinterpret_cast<const uint4*>(st_r + pp * 4 * C::STAGE_ROW);
-                    const int row = m0 + (ms * TM + t) * 32 + gq * 8 + pp * 4 + rd_r;
-                    if (row < g.M && col < g.N) *reinterpret_cast<uint4*>(out + (size_t)row * g.N + col) = val;
+                    for (int jc = 0; jc < 4; ++jc)
+#pragma unroll
+                        for (int vv = 0; vv < 4; ++vv)
+                            st_w[vv * C::STAGE_ROW + jc * 32] = E::from_f32(acc[t][cg * 4 + jc][4 * gq + vv] + bv[jc]);
+#pragma unroll
+                    for (int pp = 0; pp < 2; ++pp) {
+                        const uint4 val = *reinterpret_cast<const uint4*>(st_r + pp * 4 * C::STAGE_ROW);
+                        const int row = m0 + (ms * TM + t) * 32 + gq * 8 + pp * 4 + rd_r;
+                        if (row < g.M && col < g.N) *reinterpret_cast<uint4*>(out + (size_t)row * g.N + col) = val;
+                    }
                 }
             }
         }
     };
 
-    // same bookkeeping as the copy waves (the barriers must match), without the DMA
+    // steps whose operands have arrived from every copy wave
+    // Steps whose operands have arrived from every copy wave.  The words hold the count modulo 256 and
+    // are never more than the ring depth away from u, so the signed 8-bit difference is exact.
+    auto producers_landed = [&](int u) -> int {
+        const int v = *(const volatile int*)(s_landed + (lane & 3) * 64);
+        int m = 127;
+#pragma unroll
+        for (int c = 0; c < NP; ++c) {
+            const int d = (int)(signed char)(__builtin_amdgcn_readlane(v, c) - u);
+            m = d < m ? d : m;
+        }
+        return u + m;
+    };
     if (ns > 0) {
-        int next = 0, ent_u = 0;
-        Ends ce;
-        unpack_ends(ce, fetch_ends(0, 0));
-        while (can_issue(next, 0, 0, ce)) ++next;
         int j = 0, s = 0;
+        int landed = 0;
+        int vrec = fetch_rec(0);
         for (int u = 0; u < nsteps; ++u) {
-            if (next <= u) {
-                lds_barrier();
-                ++next;
-            }
             PBS_T(8 + 4 * u + 0);
-            const int vends = fetch_ends(j, s);
-            const int vrec = fetch_rec(s);
-            lds_barrier();
+            if (landed <= u) {
+                for (int spin = 0; spin < C::SPIN_LIMIT; ++spin) {
+                    landed = producers_landed(u);
+                    if (landed > u) break;
+                    __builtin_amdgcn_s_sleep(1);
+                }
+            }
+            asm volatile("" ::: "memory");   // operand reads stay behind the poll
             PBS_T(8 + 4 * u + 1);
-            unpack_ends(ce, vends);
-            if (u > 0)
-                while (can_issue(next, u, ent_u, ce)) ++next;
-            ent_u = ce.c0;
-            PBS_T(8 + 4 * u + 2);
-
-            // ---- the products of step s ----
             const unsigned mask = (unsigned)__builtin_amdgcn_readlane(vrec, D16_F_MASK);
             const int base = j * ne + __builtin_amdgcn_readlane(vrec, D16_F_CUM);
             const unsigned char* panel = a_ring + (u % RS) * C::PANEL_BYTES;
+            if (++s == ns) s = 0;
+            vrec = fetch_rec(s);   // the next step's record, needed after this step's products
+            PBS_T(8 + 4 * u + 2);
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk) {
                 const unsigned mk = (mask >> (16 * kk)) & 0xffffu;
@@ -475,27 +485,44 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
                 const unsigned mine = (mk >> (NBW * quarter)) & ((1u << NBW) - 1u);
 #endif
                 if (mine == 0) continue;
-                int e = base + (kk ? __popc(mask & 0xffffu) : 0) + __popc(mk & ((1u << (NBW * quarter)) - 1u));
-                uint4 fa[TM][2];
-                load_a(fa, panel, kk);
-                // the accumulator index stays static; the branches are wave-uniform
+                const int e0 = base + (kk ? __popc(mask & 0xffffu) : 0) + __popc(mk & ((1u << (NBW * quarter)) - 1u));
+                // One register index at a time keeps only 12 fragment registers live next to the 128
+                // accumulator registers.  The accumulator index stays static; the branches are wave-uniform.
 #pragma unroll
-                for (int jc = 0; jc < NBW; ++jc) {
-                    if ((mine >> jc) & 1u) {
-                        uint4 fb[2];
-                        load_b(fb, b_ring + (e & (RB - 1)) * C::BLK_BYTES);
-                        ++e;
+                for (int q = 0; q < 2; ++q) {
+                    uint4 fa[TM];
+                    load_a(fa, panel, kk, q);
+                    // The blocks of this wave's columns are consecutive entries, whichever columns they
+                    // are: the next one is fetched before the products of the current one are issued
+                    // (after the last one this reads a slot whose contents are not used).
+                    int e = e0;
+                    uint4 fb_next = load_b(b_ring + (e & (RB - 1)) * C::BLK_BYTES, q);
 #pragma unroll
-                        for (int t = 0; t < TM; ++t) E::mma(acc[t][jc], fa[t], fb);
+                    for (int jc = 0; jc < NBW; ++jc) {
+                        if ((mine >> jc) & 1u) {
+                            const uint4 fb = fb_next;
+                            ++e;
+                            fb_next = load_b(b_ring + (e & (RB - 1)) * C::BLK_BYTES, q);
+#pragma unroll
+                            for (int t = 0; t < TM; ++t)
+                                acc[t][jc] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                                    __builtin_bit_cast(bf16x8, fa[t]), __builtin_bit_cast(bf16x8, fb), acc[t][jc], 0, 0, 0);
+                        }
                     }
                 }
             }
-
+            // this wave has read everything it needs of step u: publish (steps, entries) done.  LDS
+            // serves a wave's requests in order, so the reads above precede this write.
+            asm volatile("" ::: "memory");
+            {
+                volatile int* pd = s_done + wave * 64 + lane;   // same per-lane offset as the record reads
+                pd[0] = u + 1;
+                pd[NW * 64] = base + __popc(mask);
+            }
             PBS_T(8 + 4 * u + 3);
-            if (++s == ns) {
+            if (s == 0) {
                 epilogue(j);
                 zero_acc();
-                s = 0;
                 ++j;
             }
         }

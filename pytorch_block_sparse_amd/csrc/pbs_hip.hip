@@ -62,15 +62,18 @@ static inline size_t narrow_plan_bytes(int n, int k) {
 static inline size_t wide_plan_bytes(int n, int k) {
     if (k % 64) return 0;
     const size_t groups = ((size_t)(n / 32) + D16_NB - 1) / D16_NB;
-    return groups * dds16_plan_group_ints(k / 32) * sizeof(int);
+    return (groups * dds16_plan_group_ints(k / 32) + D16_SEQ_INTS) * sizeof(int);
 }
 
-constexpr int D16_RS = 3, D16_RB = 32, D16_NP = 4;
+#ifndef PBS_EXP_D16_TM
+#define PBS_EXP_D16_TM 2
+#endif
+constexpr int D16_TM = PBS_EXP_D16_TM, D16_RS = 3, D16_RB = 32, D16_NP = 4;
 
 // Whether the wide kernel serves this problem: k-pairs need k % 64 == 0, the plan records of a group
 // must fit in LDS beside the rings, and there must be enough tiles to give every CU one.
 static bool wide_kernel_fits(long long M, int n, int k) {
-    using C = D16Cfg<D16_RS, D16_RB, D16_NP>;
+    using C = D16Cfg<D16_TM, D16_RS, D16_RB, D16_NP>;
     if (k % 64) return false;
     const size_t lds = (size_t)C::WORK_BYTES + dds16_plan_group_ints(k / 32) * sizeof(int);
     if (lds > 160 * 1024) return false;
@@ -80,9 +83,9 @@ static bool wide_kernel_fits(long long M, int n, int k) {
 
 template <int TRANS>
 static int launch_dds16(const DdsArgs& g, hipStream_t stream) {
-    using C = D16Cfg<D16_RS, D16_RB, D16_NP>;
+    using C = D16Cfg<D16_TM, D16_RS, D16_RB, D16_NP>;
     static std::atomic<uint64_t> done{0};
-    auto kernel = dds16_kernel<TRANS, D16_RS, D16_RB, D16_NP>;
+    auto kernel = dds16_kernel<TRANS, D16_TM, D16_RS, D16_RB, D16_NP>;
     D16Args a;
     a.a = g.a;
     a.data = g.data;
@@ -96,6 +99,7 @@ static int launch_dds16(const DdsArgs& g, hipStream_t stream) {
     a.m_tiles = (g.M + C::BM - 1) / C::BM;
     a.n_groups = (g.N / 32 + D16_NB - 1) / D16_NB;
     a.group_ints = (int)dds16_plan_group_ints(g.K / 32);
+    a.seq = a.plan + (size_t)a.n_groups * a.group_ints;
     // about one workgroup per CU, each walking the token tiles p, p + P, ... of its column group
     int P = 256 / a.n_groups;
     if (P < 1) P = 1;
@@ -270,7 +274,8 @@ int pbs_blocksparse_matmul_plan(const int32_t* ptr, const int32_t* indices, int 
         const int groups16 = (n / 32 + D16_NB - 1) / D16_NB;
         int* wide = reinterpret_cast<int*>(static_cast<unsigned char*>(plan) + narrow_plan_bytes(n, k));
         hipLaunchKernelGGL(dds16_plan_kernel, dim3(groups16), dim3(256), 0, static_cast<hipStream_t>(stream), ptr, indices,
-                           n / 32, k / 32, nnz, wide, (int)dds16_plan_group_ints(k / 32));
+                           n / 32, k / 32, nnz, wide, (int)dds16_plan_group_ints(k / 32),
+                           wide + (size_t)groups16 * dds16_plan_group_ints(k / 32));
     }
     return (int)hipGetLastError();
 }

@@ -10,8 +10,9 @@
 // token) and of X (16 block columns = 1 KB per token): each row is one DMA instruction
 // (global_load_lds_dwordx4, contiguous in global memory), double buffered.  The rows stay
 // token-major in LDS; both MFMA operands need 8 consecutive tokens per lane, which
-// ds_read_b64_tr_b16 gathers from 4 consecutive token rows.  To keep those 4 rows on different
-// banks the 16-byte chunks of token row t are stored at chunk position c ^ ((t & 3) << 1).
+// ds_read_b64_tr_b16 gathers from 4 consecutive token rows.  One such read takes 64 bytes from each of
+// 4 consecutive token rows per half wave; to put those on different banks the 16-byte chunks of token
+// row t are stored at chunk position c ^ ((t & 3) << 2), i.e. shifted by multiples of 64 bytes.
 //
 // Consecutive blocks of a wave mostly share their block row, so the G fragment is reloaded only
 // when the row changes.  Tokens past the end are zero rows written by the waves themselves.
@@ -107,12 +108,12 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
     const int nchunks = t_begin < t_end ? (t_end - t_begin + TC - 1) / TC : 0;
 
     // ---- DMA address pattern: this wave copies token rows wave, wave + 8, ... of both panels; the
-    //      chunk swizzle of those rows is the same ((wave & 3) << 1) ----
+    //      chunk swizzle of those rows is the same ((wave & 3) << 2) ----
     const unsigned char* G = static_cast<const unsigned char*>(a.g);
     const unsigned char* X = static_cast<const unsigned char*>(a.x);
     const int g_valid = (a.N - r0 * 32) * 2;   // bytes of a G row from this rectangle's first column on
     const int x_valid = (a.K - c0 * 32) * 2;
-    const int pc = lane ^ ((wave & 3) << 1);   // global chunk fetched by this lane
+    const int pc = lane ^ ((wave & 3) << 2);   // global chunk fetched by this lane
     const unsigned g_voff = (pc * 16 < g_valid) ? pc * 16 : 0;   // columns past the matrix edge: any valid address
     const unsigned x_voff = (pc * 16 < x_valid) ? pc * 16 : 0;
     const size_t g_row_bytes = (size_t)a.N * 2, x_row_bytes = (size_t)a.K * 2;
@@ -145,7 +146,7 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
     const int l16 = lane & 15;
     const int trow = 8 * h + (l16 >> 2);                              // + 16u + 4v
     const int cb = 2 * ((lane >> 4) & 1) + ((l16 & 3) >> 1);          // 16-byte chunk inside the block's 64 bytes
-    const int xr = ((l16 >> 2) & 3) << 1;                             // swizzle of token row trow (+ multiples of 4)
+    const int xr = ((l16 >> 2) & 3) << 2;                             // swizzle of token row trow (+ multiples of 4)
     const int lane_const = trow * C::ROW_BYTES + (l16 & 1) * 8;
     auto frag_off = [&](int blk16) -> int { return lane_const + (((blk16 * 4 + cb) ^ xr) * 16); };
 
