@@ -140,10 +140,16 @@ struct DdsArgs {
 
 // TRANS = 0: B[k][n] = block[k*32 + n]   (forward: the packed block is W_block^T = [in][out])
 // TRANS = 1: B[k][n] = block[n*32 + k]   (dX: contraction runs along the packed block's rows)
-template <typename T, int TRANS, int TM, int SK, int RS, int RB, int NP>
+template <typename T, int TRANS, int TM, int SK, int RS, int RB, int NP, int NBW_ = DDS_NBW>
 struct DdsCfg {
     using E = Elem<T>;
     static constexpr int NW = DDS_NW;                    // compute waves
+    // Block columns per compute wave: 4 (the tile covers its whole group of 8 block columns) or 2 (the
+    // tile covers half a group; twice as many, half as wide tiles for results with few columns).
+    static constexpr int NBW = NBW_;
+    static constexpr int NSUB = DDS_NBW / NBW_;          // tiles per column group
+    static constexpr int TILE_COLS = 2 * NBW_;           // block columns per tile
+    static_assert(NBW_ == 4 || NBW_ == 2, "block columns per wave");
     static constexpr int ND = NP ? NP : NW;              // waves that issue DMA
     static constexpr int NT = (NW + NP) * 64;
     static constexpr int BM = 4 * TM * 32;
@@ -161,7 +167,7 @@ struct DdsCfg {
     static constexpr int B_RING_BYTES = RB * BLK_BYTES;
     static constexpr int RING_BYTES = A_RING_BYTES + B_RING_BYTES;
     // the epilogue stages one 32-row x 128-column sub-tile per compute wave through LDS
-    static constexpr int EPI_WAVE_BYTES = 32 * 128 * E::ESZ;
+    static constexpr int EPI_WAVE_BYTES = 32 * NBW_ * 32 * E::ESZ;
     static constexpr int EPI_BYTES = NW * EPI_WAVE_BYTES;
     static constexpr int WORK_BYTES = RING_BYTES > EPI_BYTES ? RING_BYTES : EPI_BYTES;   // + the plan records
     static_assert(PANEL_INSTR % ND == 0 && A_PER_WAVE >= 1, "panel DMA must divide evenly over the issuing waves");
@@ -177,11 +183,11 @@ static __device__ __forceinline__ int swz(int r) {
     return CPR == 4 ? ((r >> 2) & 3) : ((r >> 1) & 7);
 }
 
-template <typename T, int TRANS, int TM, int SK, int RS, int RB, int NP>
+template <typename T, int TRANS, int TM, int SK, int RS, int RB, int NP, int NBW_ = DDS_NBW>
 __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
-    using C = DdsCfg<T, TRANS, TM, SK, RS, RB, NP>;
+    using C = DdsCfg<T, TRANS, TM, SK, RS, RB, NP, NBW_>;
     using E = typename C::E;
-    constexpr int NB = DDS_NB, NBW = DDS_NBW, NW = DDS_NW, ND = C::ND, NQ = E::NQ, CPR = C::CPR, R = DDS_REC_INTS;
+    constexpr int NB = DDS_NB, NBW = C::NBW, NW = DDS_NW, ND = C::ND, NQ = E::NQ, CPR = C::CPR, R = DDS_REC_INTS;
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
     unsigned char* const a_ring = smem;
@@ -190,21 +196,24 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
     const unsigned lds_a = (unsigned)(uintptr_t)a_ring;
     const unsigned lds_b = (unsigned)(uintptr_t)b_ring;
 
-    const int tile = xcd_tile_id(blockIdx.x, g.m_tiles * g.n_groups);
+    const int n_cols = g.n_groups * C::NSUB;   // tiles along the result columns
+    const int tile = xcd_tile_id(blockIdx.x, g.m_tiles * n_cols);
     if (tile < 0) return;
-    // Order of the tiles inside an XCD's range: blocks of 4 token tiles x 8 column groups, so that the
+    // Order of the tiles inside an XCD's range: blocks of 4 token tiles x 8 column tiles, so that the
     // 32 workgroups an XCD runs at a time share 4 operand panels and 8 groups of weight blocks in
     // its L2 (token-tile-major order would stream all the weights through every XCD's L2).
-    int mt, ng;
-    if ((g.n_groups % 8) == 0 && (g.m_tiles % 4) == 0) {
+    int mt, nc;
+    if ((n_cols % 8) == 0 && (g.m_tiles % 4) == 0) {
         const int blk = tile >> 5, within = tile & 31;
-        const int ngb = blk % (g.n_groups / 8), mtb = blk / (g.n_groups / 8);
+        const int ncb = blk % (n_cols / 8), mtb = blk / (n_cols / 8);
         mt = mtb * 4 + (within >> 3);
-        ng = ngb * 8 + (within & 7);
+        nc = ncb * 8 + (within & 7);
     } else {
-        mt = tile / g.n_groups;
-        ng = tile % g.n_groups;
+        mt = tile / n_cols;
+        nc = tile % n_cols;
     }
+    const int ng = nc / C::NSUB;                        // column group (plan records)
+    const int col_lo = (nc % C::NSUB) * C::TILE_COLS;   // first of this tile's columns within the group
     const int m0 = mt * C::BM;
     const int nb0 = ng * NB;
 
@@ -316,7 +325,7 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
 #pragma unroll
                 for (int c = 0; c < C::COLS_PER_COPIER; ++c) {
                     const int j = dw + c * ND;
-                    if ((mask >> j) & 1) {
+                    if (((mask >> j) & 1) && (C::NSUB == 1 || (j >= col_lo && j < col_lo + C::TILE_COLS))) {
                         const int e = base + __popc(mask & ((1 << j) - 1));
                         const unsigned char* bsrc =
                             uniform_ptr(D + (size_t)__builtin_amdgcn_readlane(vrec, k * R + j) * C::BLK_BYTES);
@@ -398,7 +407,8 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
     // compute side
     // =====================================================================================
     const int ms = wave & 3;            // token slice
-    const int half = (wave >> 2) & 1;   // block-column half
+    const int half = (wave >> 2) & 1;   // block-column half of the tile
+    const int col_w = col_lo + half * NBW;   // first of this wave's columns within the group
     const int lrow = lane & 31;
     const int h = lane >> 5;
 
@@ -475,9 +485,9 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
 #pragma unroll
         for (int k = 0; k < SK; ++k) {
             const int mask = st_mask[k];
-            const int mine = (mask >> (NBW * half)) & ((1 << NBW) - 1);
+            const int mine = (mask >> col_w) & ((1 << NBW) - 1);
             if (mine == 0) continue;
-            int e = st_cum[k] + (half ? __popc(mask & ((1 << NBW) - 1)) : 0);
+            int e = st_cum[k] + __popc(mask & ((1 << col_w) - 1));
             uint4 fa[TM][NQ];
             load_a(fa, stage + k * C::PANEL_BYTES);
             // the accumulator index stays static; the branches are wave-uniform
@@ -534,7 +544,7 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
     T* out = static_cast<T*>(g.out);
     const T* bias = static_cast<const T*>(g.bias);
     unsigned char* epi = smem + wave * C::EPI_WAVE_BYTES;
-    const int col0 = (nb0 + half * NBW) * 32;             // first column of this wave's half
+    const int col0 = (nb0 + col_w) * 32;                  // first result column of this wave
     float bv[NBW];
 #pragma unroll
     for (int j = 0; j < NBW; ++j) {
@@ -542,7 +552,8 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
         bv[j] = (bias && col < g.N) ? E::to_f32(bias[col]) : 0.f;
     }
     constexpr int EPL = 16 / E::ESZ;                       // elements per 16-byte chunk
-    constexpr int CHUNKS_PER_ROW = 128 / EPL;              // 16 (bf16) or 32 (fp32)
+    constexpr int WCOLS = NBW * 32;                        // result columns of one wave
+    constexpr int CHUNKS_PER_ROW = WCOLS / EPL;            // 16-byte chunks per staged row
     constexpr int ROWS_PER_PASS = 64 / CHUNKS_PER_ROW;     // rows stored by one wave instruction
 #pragma unroll
     for (int t = 0; t < TM; ++t) {
@@ -550,14 +561,14 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
 #pragma unroll
         for (int j = 0; j < NBW; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) e_t[acc_row(v, h) * 128 + j * 32 + lrow] = E::from_f32(acc[t][j][v] + bv[j]);
+            for (int v = 0; v < 16; ++v) e_t[acc_row(v, h) * WCOLS + j * 32 + lrow] = E::from_f32(acc[t][j][v] + bv[j]);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         const int rbase = m0 + (ms * TM + t) * 32;
 #pragma unroll
         for (int p = 0; p < 32 / ROWS_PER_PASS; ++p) {
             const int r = p * ROWS_PER_PASS + lane / CHUNKS_PER_ROW;
             const int c = (lane % CHUNKS_PER_ROW) * EPL;
-            const uint4 val = *reinterpret_cast<const uint4*>(epi + (r * 128 + c) * E::ESZ);
+            const uint4 val = *reinterpret_cast<const uint4*>(epi + (r * WCOLS + c) * E::ESZ);
             const int row = rbase + r, col = col0 + c;
             if (row < g.M && col < g.N) *reinterpret_cast<uint4*>(out + (size_t)row * g.N + col) = val;
         }

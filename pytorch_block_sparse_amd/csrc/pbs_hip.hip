@@ -36,18 +36,18 @@ static int raise_lds_limit(K kernel, int bytes, std::atomic<uint64_t>& done) {
     return 0;
 }
 
-template <typename T, int TRANS, int TM, int SK, int RS, int RB, int NP>
+template <typename T, int TRANS, int TM, int SK, int RS, int RB, int NP, int NBW = DDS_NBW>
 static int launch_dds(DdsArgs g, hipStream_t stream) {
-    using C = DdsCfg<T, TRANS, TM, SK, RS, RB, NP>;
+    using C = DdsCfg<T, TRANS, TM, SK, RS, RB, NP, NBW>;
     static std::atomic<uint64_t> done{0};
-    auto kernel = dds_kernel<T, TRANS, TM, SK, RS, RB, NP>;
+    auto kernel = dds_kernel<T, TRANS, TM, SK, RS, RB, NP, NBW>;
     constexpr int LDS_MAX = 160 * 1024;
     // rings (or the epilogue staging) plus this group's plan records
     const size_t lds = (size_t)C::WORK_BYTES + (size_t)g.group_ints * sizeof(int);
     if (lds > (size_t)LDS_MAX) return PBS_ERR_TOO_LARGE;
     if (int rc = raise_lds_limit(kernel, LDS_MAX, done)) return rc;
     g.m_tiles = (g.M + C::BM - 1) / C::BM;
-    const long long tiles = (long long)g.m_tiles * g.n_groups;
+    const long long tiles = (long long)g.m_tiles * g.n_groups * C::NSUB;
     if (tiles > (1ll << 30)) return PBS_ERR_TOO_LARGE;
     hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)tiles)), dim3(C::NT), lds, stream, g);
     return (int)hipGetLastError();
@@ -113,22 +113,22 @@ static int launch_dds16(const DdsArgs& g, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
-// Tile shapes: 256 tokens x 8 block columns when that still gives every CU a tile, else 128 tokens.
+// Tile shapes: 256 tokens x 8 block columns when that still gives every CU a tile, else 128 tokens x 8,
+// else (results with few columns) 128 tokens x 4 block columns.
 // bf16 steps cover two k-blocks (the matrix cores go through a k-block 16x faster than in fp32).
 template <typename T, int TRANS>
 static int dispatch_dds(const DdsArgs& g, hipStream_t stream) {
     const long long big_tiles = (long long)((g.M + 255) / 256) * g.n_groups;
+    const long long mid_tiles = (long long)((g.M + 127) / 128) * g.n_groups;
     if constexpr (sizeof(T) == 4) {
         if (big_tiles >= 256) return launch_dds<T, TRANS, 2, 1, 3, 8, 0>(g, stream);
-        return launch_dds<T, TRANS, 1, 1, 3, 8, 0>(g, stream);
+        if (mid_tiles >= 160) return launch_dds<T, TRANS, 1, 1, 3, 8, 0>(g, stream);
+        return launch_dds<T, TRANS, 1, 1, 3, 8, 0, 2>(g, stream);
     } else {
-#ifdef PBS_EXP_BF16_CFG
-        return launch_dds<T, TRANS, PBS_EXP_BF16_CFG>(g, stream);
-#else
         if (wide_kernel_fits(g.M, g.N, g.K)) return launch_dds16<TRANS>(g, stream);
         if (big_tiles >= 256) return launch_dds<T, TRANS, 2, 2, 3, 16, 4>(g, stream);
-        return launch_dds<T, TRANS, 1, 2, 3, 16, 4>(g, stream);
-#endif
+        if (mid_tiles >= 160) return launch_dds<T, TRANS, 1, 2, 3, 16, 4>(g, stream);
+        return launch_dds<T, TRANS, 1, 2, 3, 16, 4, 2>(g, stream);
     }
 }
 
@@ -152,8 +152,9 @@ static SddPlan plan_sdd(long long M, int N, int K, int SR, int SC, int TC) {
     p.tiles_c = (K / 32 + SC - 1) / SC;
     const long long tiles = (long long)p.tiles_r * p.tiles_c;
     const long long chunks = (M + TC - 1) / TC;
-    // aim at one or two workgroups per CU, but keep at least 8 chunks of tokens per slice
-    long long want = (256 + tiles - 1) / tiles;
+    // Aim at one workgroup per CU and never slightly more (the kernels' registers and LDS allow one
+    // workgroup per CU, so 257 workgroups take twice as long as 256); keep at least 8 chunks per slice.
+    long long want = 256 / tiles;
     long long cap = chunks / 8;
     if (cap < 1) cap = 1;
     if (want > cap) want = cap;
