@@ -44,42 +44,96 @@ constexpr int DDS_NBW = 4;   // block columns per compute wave
 constexpr int DDS_NW = 8;    // compute waves per workgroup: 4 token slices x 2 column halves
 
 // ---- plan layout per group of DDS_NB block columns: (KB + 2) records of 16 ints (KB = K/32) ----
-//   record 0        header: [0] = nk (present k-blocks), [1] = ne (entries)
+//   record 0        header: [0] = nk (present k-blocks), [1] = ne (entries), [2..9] = block column of the
+//                   result in each of the group's 8 places, or -1
 //   record 1 + i    i-th present k-block: [0..7] data block of each column or -1,
 //                   [8] k-block, [9] present-column mask, [10] entries before it
 //   record 1 + nk   sentinel: [10] = ne
 constexpr int DDS_REC_INTS = 16;
 constexpr int DDS_F_KB = 8, DDS_F_MASK = 9, DDS_F_CUM = 10;
+constexpr int DDS_H_COL = 2;
 static inline size_t dds_plan_group_ints(int KB) { return ((size_t)KB + 2) * DDS_REC_INTS; }
+
+// Which block columns of the result form a group.  Normally group g is columns 8g .. 8g+7.  When the
+// per-column block counts are very uneven (largest > 2x the mean) the columns are ranked by count
+// and dealt to the half-groups of 4 in serpentine order, so every tile gets about the same number
+// of blocks: a tile of a few heavy columns would otherwise run long after all others are done.
+// slots[8g + j] = block column in place j of group g, or -1.  One workgroup.
+constexpr int DDS_BALANCE_MAX_COLS = 4096;
+__global__ __launch_bounds__(256) void dds_slots_kernel(const int32_t* __restrict__ ptr, int nblk_n, int n_groups,
+                                                        int* slots) {
+    constexpr int NT = 256;
+    __shared__ int s_cnt[DDS_BALANCE_MAX_COLS];
+    __shared__ int s_slot[DDS_BALANCE_MAX_COLS + DDS_NB];
+    __shared__ int s_max, s_sum;
+    const int tid = threadIdx.x;
+    const int total = n_groups * DDS_NB;
+    bool skewed = false;
+    if (nblk_n <= DDS_BALANCE_MAX_COLS && n_groups >= 2) {
+        if (tid == 0) {
+            s_max = 0;
+            s_sum = 0;
+        }
+        __syncthreads();
+        for (int c = tid; c < nblk_n; c += NT) {
+            const int n = ptr[c + 1] - ptr[c];
+            s_cnt[c] = n;
+            atomicMax(&s_max, n);
+            atomicAdd(&s_sum, n);
+        }
+        __syncthreads();
+        skewed = (long long)s_max * nblk_n > 2ll * s_sum;
+    }
+    if (!skewed) {
+        for (int i = tid; i < total; i += NT) slots[i] = i < nblk_n ? i : -1;
+        return;
+    }
+    for (int i = tid; i < total; i += NT) s_slot[i] = -1;
+    __syncthreads();
+    const int units = 2 * n_groups;   // half-groups of 4 columns
+    for (int c = tid; c < nblk_n; c += NT) {
+        const int n = s_cnt[c];
+        int rank = 0;
+        for (int o = 0; o < nblk_n; ++o) {
+            const int m = s_cnt[o];
+            rank += (m > n || (m == n && o < c)) ? 1 : 0;
+        }
+        const int place = rank / units;            // 0..3 within the half-group
+        int u = rank % units;
+        if (place & 1) u = units - 1 - u;          // serpentine: heavy and light columns pair up
+        s_slot[(u >> 1) * DDS_NB + (u & 1) * 4 + place] = c;
+    }
+    __syncthreads();
+    for (int i = tid; i < total; i += NT) slots[i] = s_slot[i];
+}
 
 // One workgroup per group of 8 block columns merges their sorted block lists.
 __global__ __launch_bounds__(256) void dds_plan_kernel(const int32_t* __restrict__ ptr, const int32_t* __restrict__ idx,
-                                                       int nblk_n, int KB, int nnz, int* plan, int group_ints) {
+                                                       const int* __restrict__ slots, int nblk_n, int KB, int nnz,
+                                                       int* plan, int group_ints) {
     constexpr int NB = DDS_NB, SEG = 128, NT = 256, R = DDS_REC_INTS;
     __shared__ int s_tbl[SEG * NB];
-    __shared__ int s_ptr[NB + 1];
+    __shared__ int s_lo[NB], s_hi[NB], s_col[NB];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int nb0 = blockIdx.x * NB;
     int* out = plan + (size_t)blockIdx.x * group_ints;
     int* rec = out + R;
-    if (tid <= NB) {
-        const int nb = nb0 + tid;
-        s_ptr[tid] = ptr[nb < nblk_n ? nb : nblk_n];
+    if (tid < NB) {
+        const int c = slots[blockIdx.x * NB + tid];
+        const bool ok = c >= 0 && c < nblk_n;
+        s_col[tid] = ok ? c : -1;
+        s_lo[tid] = ok ? ptr[c] : 0;
+        s_hi[tid] = ok ? ptr[c + 1] : 0;
     }
     __syncthreads();
-    const int e_begin = s_ptr[0], e_end = s_ptr[NB];
     int nk = 0, ne = 0;   // running totals (kept by every thread of wave 0)
     for (int seg0 = 0; seg0 < KB; seg0 += SEG) {
         for (int i = tid; i < SEG * NB; i += NT) s_tbl[i] = -1;
         __syncthreads();
-        for (int e = e_begin + tid; e < e_end; e += NT) {
-            const int kb = idx[2 * e] - seg0;
-            const int b = idx[2 * e + 1];
-            if (kb >= 0 && kb < SEG && kb + seg0 < KB && b >= 0 && b < nnz) {
-                int nl = 0;
-#pragma unroll
-                for (int i = 1; i < NB; ++i) nl += (e >= s_ptr[i]) ? 1 : 0;
-                s_tbl[kb * NB + nl] = b;
+        for (int jc = 0; jc < NB; ++jc) {
+            for (int e = s_lo[jc] + tid; e < s_hi[jc]; e += NT) {
+                const int kb = idx[2 * e] - seg0;
+                const int b = idx[2 * e + 1];
+                if (kb >= 0 && kb < SEG && kb + seg0 < KB && b >= 0 && b < nnz) s_tbl[kb * NB + jc] = b;
             }
         }
         __syncthreads();
@@ -115,7 +169,12 @@ __global__ __launch_bounds__(256) void dds_plan_kernel(const int32_t* __restrict
         __syncthreads();
     }
     if (wave == 0 && lane < R) {
-        out[lane] = lane == 0 ? nk : (lane == 1 ? ne : 0);
+        // header: counts, then the block column in each of the group's 8 places
+        int hv = 0;
+        if (lane == 0) hv = nk;
+        else if (lane == 1) hv = ne;
+        else if (lane >= DDS_H_COL && lane < DDS_H_COL + NB) hv = s_col[lane - DDS_H_COL];
+        out[lane] = hv;
         int* r = rec + (size_t)nk * R;   // sentinel
         r[lane] = lane < NB ? -1 : (lane == DDS_F_CUM ? ne : 0);
     }
@@ -187,7 +246,7 @@ template <typename T, int TRANS, int TM, int SK, int RS, int RB, int NP, int NBW
 __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
     using C = DdsCfg<T, TRANS, TM, SK, RS, RB, NP, NBW_>;
     using E = typename C::E;
-    constexpr int NB = DDS_NB, NBW = C::NBW, NW = DDS_NW, ND = C::ND, NQ = E::NQ, CPR = C::CPR, R = DDS_REC_INTS;
+    constexpr int NBW = C::NBW, NW = DDS_NW, ND = C::ND, NQ = E::NQ, CPR = C::CPR, R = DDS_REC_INTS;
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
     unsigned char* const a_ring = smem;
@@ -215,7 +274,6 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
     const int ng = nc / C::NSUB;                        // column group (plan records)
     const int col_lo = (nc % C::NSUB) * C::TILE_COLS;   // first of this tile's columns within the group
     const int m0 = mt * C::BM;
-    const int nb0 = ng * NB;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -544,12 +602,13 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
     T* out = static_cast<T*>(g.out);
     const T* bias = static_cast<const T*>(g.bias);
     unsigned char* epi = smem + wave * C::EPI_WAVE_BYTES;
-    const int col0 = (nb0 + col_w) * 32;                  // first result column of this wave
+    int colid[NBW];   // block columns of the result this wave owns (-1: none)
+#pragma unroll
+    for (int j = 0; j < NBW; ++j) colid[j] = __builtin_amdgcn_readfirstlane(s_plan[DDS_H_COL + col_w + j]);
     float bv[NBW];
 #pragma unroll
     for (int j = 0; j < NBW; ++j) {
-        const int col = col0 + j * 32 + lrow;
-        bv[j] = (bias && col < g.N) ? E::to_f32(bias[col]) : 0.f;
+        bv[j] = (bias && colid[j] >= 0) ? E::to_f32(bias[colid[j] * 32 + lrow]) : 0.f;
     }
     constexpr int EPL = 16 / E::ESZ;                       // elements per 16-byte chunk
     constexpr int WCOLS = NBW * 32;                        // result columns of one wave
@@ -569,8 +628,11 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
             const int r = p * ROWS_PER_PASS + lane / CHUNKS_PER_ROW;
             const int c = (lane % CHUNKS_PER_ROW) * EPL;
             const uint4 val = *reinterpret_cast<const uint4*>(epi + (r * WCOLS + c) * E::ESZ);
-            const int row = rbase + r, col = col0 + c;
-            if (row < g.M && col < g.N) *reinterpret_cast<uint4*>(out + (size_t)row * g.N + col) = val;
+            int cid = colid[0];   // the block column this lane's chunk belongs to
+#pragma unroll
+            for (int j = 1; j < NBW; ++j) cid = (c >= j * 32) ? colid[j] : cid;
+            const int row = rbase + r, col = cid * 32 + (c & 31);
+            if (row < g.M && cid >= 0) *reinterpret_cast<uint4*>(out + (size_t)row * g.N + col) = val;
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }

@@ -59,6 +59,10 @@ static inline size_t narrow_plan_bytes(int n, int k) {
     const size_t groups = ((size_t)(n / 32) + DDS_NB - 1) / DDS_NB;
     return groups * dds_plan_group_ints(k / 32) * sizeof(int);
 }
+static inline size_t slot_table_bytes(int n) {   // behind the plans: the block column in every place of every group
+    const size_t groups = ((size_t)(n / 32) + DDS_NB - 1) / DDS_NB;
+    return ((groups * DDS_NB * sizeof(int)) + 63) / 64 * 64;
+}
 static inline size_t wide_plan_bytes(int n, int k) {
     if (k % 64) return 0;
     const size_t groups = ((size_t)(n / 32) + D16_NB - 1) / D16_NB;
@@ -258,7 +262,7 @@ int pbs_build_indices(const uint8_t* mask, const int64_t* block_ptr, int X, int 
 
 size_t pbs_blocksparse_matmul_plan_bytes(int n, int k) {
     if (n <= 0 || k <= 0 || (n % 32) || (k % 32)) return 0;
-    return narrow_plan_bytes(n, k) + wide_plan_bytes(n, k);
+    return narrow_plan_bytes(n, k) + wide_plan_bytes(n, k) + slot_table_bytes(n);
 }
 
 int pbs_blocksparse_matmul_plan(const int32_t* ptr, const int32_t* indices, int n, int k, int nnz, void* plan,
@@ -268,8 +272,11 @@ int pbs_blocksparse_matmul_plan(const int32_t* ptr, const int32_t* indices, int 
     if (!ptr || !plan || (nnz > 0 && !indices)) return PBS_ERR_NULL_POINTER;
     if (!aligned16(plan) || plan_bytes < pbs_blocksparse_matmul_plan_bytes(n, k)) return PBS_ERR_WORKSPACE;
     const int groups = (n / 32 + DDS_NB - 1) / DDS_NB;
-    hipLaunchKernelGGL(dds_plan_kernel, dim3(groups), dim3(256), 0, static_cast<hipStream_t>(stream), ptr, indices, n / 32,
-                       k / 32, nnz, static_cast<int*>(plan), (int)dds_plan_group_ints(k / 32));
+    int* slots = reinterpret_cast<int*>(static_cast<unsigned char*>(plan) + narrow_plan_bytes(n, k) + wide_plan_bytes(n, k));
+    hipLaunchKernelGGL(dds_slots_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(stream), ptr, n / 32, groups, slots);
+    if (int rc = (int)hipGetLastError()) return rc;
+    hipLaunchKernelGGL(dds_plan_kernel, dim3(groups), dim3(256), 0, static_cast<hipStream_t>(stream), ptr, indices, slots,
+                       n / 32, k / 32, nnz, static_cast<int*>(plan), (int)dds_plan_group_ints(k / 32));
     if (int rc = (int)hipGetLastError()) return rc;
     if (wide_plan_bytes(n, k)) {
         const int groups16 = (n / 32 + D16_NB - 1) / D16_NB;

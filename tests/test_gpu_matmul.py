@@ -219,3 +219,21 @@ def test_benchmark_config_bf16_4096_tokens(cuda):
     assert_close(m.reverse_matmul(xd, True), y_ref, w.dtype, "c4/4096 fwd")
     assert_close(m.reverse_matmul(dyd, False), dx_ref, w.dtype, "c4/4096 dx")
     assert_close(m.matmul_with_output_sparse_support(dyd, xd), dw_ref, w.dtype, "c4/4096 dw")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_uneven_rows_use_balanced_column_groups(cuda, dtype):
+    """Very uneven block counts per row of W (and, transposed, per column): the result's block columns
+    are regrouped by count.  Values, the fused bias and untouched columns must not notice."""
+    out_f, in_f, tokens = 13 * 32, 10 * 32, 300
+    blocks = [(0, c) for c in range(10)] + [(1, c) for c in range(0, 10, 2)] + [(r, (3 * r) % 10) for r in range(2, 12)]
+    m = _matrix(out_f, in_f, blocks, None, dtype, cuda, seed=13)   # block row 12 of W is empty
+    _check_all(m, (tokens,), dtype, cuda, 17, "uneven rows")
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn((tokens, in_f), generator=g).to(dtype)
+    bias = torch.randn((out_f,), generator=g).to(dtype)
+    coo = m.build_coo_block_index().cpu().numpy()
+    w_dense = O.to_dense(to64(m.data), coo, (out_f, in_f))
+    yb = m.reverse_matmul(x.to(cuda), True, bias=bias.to(cuda))
+    assert_close(yb, to64(x) @ w_dense.T + to64(bias)[None, :], dtype, "uneven rows fwd + bias")
+    assert torch.equal(yb[:, 12 * 32:], bias.to(cuda)[None, 12 * 32:].expand(tokens, -1))
