@@ -25,6 +25,55 @@ struct SddArgs {
     int tokens_per_split;    // multiple of TC
 };
 
+// Which block rows of W form row band `band` of rectangles (SR places; -1 = no row).  Normally they are
+// rows SR*band .. SR*band + SR - 1.  When the per-row block counts are very uneven (largest > 2x the
+// mean) the rows are ranked by count and dealt to the bands in serpentine order, so that all
+// rectangles hold about the same number of blocks.  Every workgroup derives its own band from the
+// row pointer array (a few microseconds at most; above SDD_BALANCE_MAX_ROWS rows the natural order
+// is kept).  Called by all threads of the workgroup; `scratch` is LDS for nblk_r + 2 ints.
+constexpr int SDD_BALANCE_MAX_ROWS = 1024;
+static __device__ __forceinline__ void sdd_band_rows(const int32_t* __restrict__ ptr, int nblk_r, int tiles_r, int band,
+                                                     int SR, int* s_rowid, int* scratch, int tid, int nthreads) {
+    bool skewed = false;
+    if (nblk_r <= SDD_BALANCE_MAX_ROWS && tiles_r >= 2) {
+        int* s_max = scratch + nblk_r;
+        int* s_sum = s_max + 1;
+        if (tid == 0) {
+            *s_max = 0;
+            *s_sum = 0;
+        }
+        __syncthreads();
+        for (int r = tid; r < nblk_r; r += nthreads) {
+            const int n = ptr[r + 1] - ptr[r];
+            scratch[r] = n;
+            atomicMax(s_max, n);
+            atomicAdd(s_sum, n);
+        }
+        __syncthreads();
+        skewed = (long long)*s_max * nblk_r > 2ll * *s_sum;
+    }
+    if (tid < SR) {
+        const int r = band * SR + tid;
+        s_rowid[tid] = (!skewed && r < nblk_r) ? r : -1;
+    }
+    __syncthreads();
+    if (skewed) {
+        for (int r = tid; r < nblk_r; r += nthreads) {
+            const int n = scratch[r];
+            int rank = 0;
+            for (int o = 0; o < nblk_r; ++o) {
+                const int m = scratch[o];
+                rank += (m > n || (m == n && o < r)) ? 1 : 0;
+            }
+            const int place = rank / tiles_r;
+            int b = rank % tiles_r;
+            if (place & 1) b = tiles_r - 1 - b;
+            if (b == band && place < SR) s_rowid[place] = r;
+        }
+        __syncthreads();
+    }
+}
+
 template <typename T, int SR, int SC, int QW, int NW>
 struct SddCfg {
     using E = Elem<T>;
@@ -71,7 +120,6 @@ __global__ __launch_bounds__(NW * 64) void sdd_kernel(SddArgs a) {
     const int tile = wg % ntiles;
     const int tr = tile / a.tiles_c;
     const int tc = tile % a.tiles_c;
-    const int r0 = tr * SR;
     const int c0 = tc * SC;
     const int nblk_r = a.N / 32;
 
@@ -83,9 +131,11 @@ __global__ __launch_bounds__(NW * 64) void sdd_kernel(SddArgs a) {
 
     // ---- list the nonzero blocks of the rectangle, row-major ----
     int my_lo = 0, my_n = 0;
+    __shared__ int s_rowid[SR];   // block row of W in each place of this rectangle's band, or -1
+    sdd_band_rows(a.ptr, nblk_r, a.tiles_r, tr, SR, s_rowid, reinterpret_cast<int*>(smem), tid, NT);
     if (tid < SR) {
-        const int r = r0 + tid;
-        if (r < nblk_r) {
+        const int r = s_rowid[tid];
+        if (r >= 0) {
             int lo = a.ptr[r], hi = a.ptr[r + 1];
             // rows are sorted by block column: first entry with column >= c0
             int l = lo, u = hi;
@@ -132,10 +182,13 @@ __global__ __launch_bounds__(NW * 64) void sdd_kernel(SddArgs a) {
 
     const unsigned char* G = static_cast<const unsigned char*>(a.g);
     const unsigned char* X = static_cast<const unsigned char*>(a.x);
-    const size_t g_col0 = (size_t)r0 * 32 * E::ESZ;
     const size_t x_col0 = (size_t)c0 * 32 * E::ESZ;
-    const int g_valid = (a.N - r0 * 32) * E::ESZ;   // bytes of a G row that exist from column r0*32 on
     const int x_valid = (a.K - c0 * 32) * E::ESZ;
+    // byte offset, inside a G row, of the 16-byte piece at panel byte cb (-1: that block row does not exist)
+    auto g_piece = [&](int cb) -> int {
+        const int rid = s_rowid[cb / (32 * E::ESZ)];
+        return rid < 0 ? -1 : rid * 32 * E::ESZ + cb % (32 * E::ESZ);
+    };
 
     uint4 rg[C::NG];
     uint4 rx[C::NX];
@@ -145,13 +198,26 @@ __global__ __launch_bounds__(NW * 64) void sdd_kernel(SddArgs a) {
         if (t < t_end && cb < valid) return ldg16(base + (size_t)t * ld_bytes + col0 + cb);
         return make_uint4(0, 0, 0, 0);
     };
+    auto ld_g = [&](size_t ld_bytes, int t, int piece) -> uint4 {
+        if (t < t_end && piece >= 0) return ldg16(G + (size_t)t * ld_bytes + piece);
+        return make_uint4(0, 0, 0, 0);
+    };
+    // the G pieces a thread stages are the same in every chunk
+    int g_off[C::NG];
+    if constexpr (E::ESZ == 4) {
+#pragma unroll
+        for (int i = 0; i < C::NG; ++i) g_off[i] = g_piece(((i * NT + tid) % (FG / 4)) * 16);
+    } else {
+#pragma unroll
+        for (int i = 0; i < C::NG / 2; ++i) g_off[i] = g_piece(((i * NT + tid) % (FG / 8)) * 16);
+    }
     auto load_chunk = [&](int ci) {
         const int t0 = t_begin + ci * TC;
         if constexpr (E::ESZ == 4) {
 #pragma unroll
             for (int i = 0; i < C::NG; ++i) {
                 const int q = i * NT + tid;
-                rg[i] = ld_panel(G, (size_t)a.N * 4, g_col0, g_valid, t0 + q / (FG / 4), (q % (FG / 4)) * 16);
+                rg[i] = ld_g((size_t)a.N * 4, t0 + q / (FG / 4), g_off[i]);
             }
 #pragma unroll
             for (int i = 0; i < C::NX; ++i) {
@@ -164,8 +230,9 @@ __global__ __launch_bounds__(NW * 64) void sdd_kernel(SddArgs a) {
             for (int i = 0; i < C::NG / 2; ++i) {
                 const int u = i * NT + tid;
                 const int tp = u / (FG / 8), f8 = u % (FG / 8);
-                rg[2 * i] = ld_panel(G, (size_t)a.N * 2, g_col0, g_valid, t0 + 2 * tp, f8 * 16);
-                rg[2 * i + 1] = ld_panel(G, (size_t)a.N * 2, g_col0, g_valid, t0 + 2 * tp + 1, f8 * 16);
+                (void)f8;
+                rg[2 * i] = ld_g((size_t)a.N * 2, t0 + 2 * tp, g_off[i]);
+                rg[2 * i + 1] = ld_g((size_t)a.N * 2, t0 + 2 * tp + 1, g_off[i]);
             }
 #pragma unroll
             for (int i = 0; i < C::NX / 2; ++i) {

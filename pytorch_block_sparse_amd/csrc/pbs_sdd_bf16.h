@@ -30,7 +30,7 @@ struct SddBf16Cfg {
     static constexpr int STAGE_BYTES = 2 * PANEL_BYTES;      // G panel, then X panel
     static constexpr int LIST_MAX = SR * SC;
     static constexpr int QMAX = QW * NW;
-    static constexpr int LDS_BYTES = 2 * STAGE_BYTES + LIST_MAX * 4 + LIST_MAX * 2 + (SR + 4) * 4;
+    static constexpr int LDS_BYTES = 2 * STAGE_BYTES + LIST_MAX * 4 + LIST_MAX * 2 + (2 * SR + 4) * 4;
     static constexpr int ROWS_PER_WAVE = TC / NW;            // token rows of each panel a wave copies per chunk
 };
 
@@ -50,7 +50,6 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
     if (wg < 0) return;
     const int sp = wg / ntiles;
     const int tile = wg % ntiles;
-    const int r0 = (tile / a.tiles_c) * SR;
     const int c0 = (tile % a.tiles_c) * SC;
     const int nblk_r = a.N / 32;
 
@@ -61,10 +60,12 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
     const int h = lane >> 5;
 
     // ---- list the blocks of the rectangle, row-major ----
+    int* s_rowid = s_rowoff + SR + 2;   // [SR] block row of W in each place of this rectangle's band, or -1
     int my_lo = 0, my_n = 0;
+    sdd_band_rows(a.ptr, nblk_r, a.tiles_r, tile / a.tiles_c, SR, s_rowid, reinterpret_cast<int*>(smem), tid, C::NT);
     if (tid < SR) {
-        const int r = r0 + tid;
-        if (r < nblk_r) {
+        const int r = s_rowid[tid];
+        if (r >= 0) {
             const int lo = a.ptr[r], hi = a.ptr[r + 1];
             int l = lo, u = hi;
             while (l < u) {   // rows are sorted by block column: first entry with column >= c0
@@ -111,13 +112,15 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
     //      chunk swizzle of those rows is the same ((wave & 3) << 2) ----
     const unsigned char* G = static_cast<const unsigned char*>(a.g);
     const unsigned char* X = static_cast<const unsigned char*>(a.x);
-    const int g_valid = (a.N - r0 * 32) * 2;   // bytes of a G row from this rectangle's first column on
     const int x_valid = (a.K - c0 * 32) * 2;
-    const int pc = lane ^ ((wave & 3) << 2);   // global chunk fetched by this lane
-    const unsigned g_voff = (pc * 16 < g_valid) ? pc * 16 : 0;   // columns past the matrix edge: any valid address
+    const int pc = lane ^ ((wave & 3) << 2);   // panel chunk fetched by this lane
+    // G: the 64 bytes of place pc / 4 of the band come from that place's block row (a place without a
+    // row fetches any valid address; nothing reads it)
+    const int g_rid = s_rowid[pc >> 2];
+    const unsigned g_voff = g_rid >= 0 ? (unsigned)(g_rid * 64 + (pc & 3) * 16) : 0u;
     const unsigned x_voff = (pc * 16 < x_valid) ? pc * 16 : 0;
     const size_t g_row_bytes = (size_t)a.N * 2, x_row_bytes = (size_t)a.K * 2;
-    const unsigned char* g_col = G + (size_t)r0 * 64;
+    const unsigned char* g_col = G;
     const unsigned char* x_col = X + (size_t)c0 * 64;
 
     auto issue_chunk = [&](int ci) {
