@@ -142,8 +142,12 @@ static int dispatch_dds(const DdsArgs& g, hipStream_t stream) {
 struct SddShapeF32 {
     static constexpr int SR = 8, SC = 8, QW = 8, NW = 4, TC = 16;
 };
+#ifndef PBS_EXP_SDD_TC
+#define PBS_EXP_SDD_TC 32
+#define PBS_EXP_SDD_NS 2
+#endif
 struct SddShapeBf16 {
-    static constexpr int SR = 16, SC = 16, QW = 10, TC = 32;
+    static constexpr int SR = 16, SC = 16, QW = 10, TC = PBS_EXP_SDD_TC, NS = PBS_EXP_SDD_NS;
 };
 
 struct SddPlan {
@@ -200,10 +204,10 @@ static int launch_sdd(SddArgs a, int dtype, void* workspace, size_t workspace_by
         hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)wgs)), dim3(C::NT), C::LDS_BYTES, stream, a);
     } else {
         using S = SddShapeBf16;
-        using C = SddBf16Cfg<S::QW>;
+        using C = SddBf16Cfg<S::QW, S::TC, S::NS>;
         static_assert(C::TC == S::TC && C::SR == S::SR && C::SC == S::SC, "plan and kernel must agree");
         static std::atomic<uint64_t> done{0};
-        auto kernel = sdd_bf16_kernel<S::QW>;
+        auto kernel = sdd_bf16_kernel<S::QW, S::TC, S::NS>;
         if (int rc = raise_lds_limit(kernel, C::LDS_BYTES, done)) return rc;
         hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)wgs)), dim3(C::NT), C::LDS_BYTES, stream, a);
     }

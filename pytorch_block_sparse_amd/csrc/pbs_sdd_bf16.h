@@ -8,7 +8,9 @@
 //
 // Tokens are streamed in chunks of 32.  A chunk is 32 token rows of G (16 block rows = 1 KB per
 // token) and of X (16 block columns = 1 KB per token): each row is one DMA instruction
-// (global_load_lds_dwordx4, contiguous in global memory), double buffered.  The rows stay
+// (global_load_lds_dwordx4, contiguous in global memory) into one of NS chunk buffers, so that NS - 1
+// chunks of loads are in flight while one is consumed (the operands come from HBM; a single chunk in
+// flight does not cover that latency).  The rows stay
 // token-major in LDS; both MFMA operands need 8 consecutive tokens per lane, which
 // ds_read_b64_tr_b16 gathers from 4 consecutive token rows.  One such read takes 64 bytes from each of
 // 4 consecutive token rows per half wave; to put those on different banks the 16-byte chunks of token
@@ -22,25 +24,30 @@
 
 namespace pbs {
 
-template <int QW>
+template <int QW, int TC_, int NS_>
 struct SddBf16Cfg {
-    static constexpr int SR = 16, SC = 16, NW = 8, NT = NW * 64, TC = 32;
+    static constexpr int SR = 16, SC = 16, NW = 8, NT = NW * 64;
+    static constexpr int TC = TC_;                           // tokens per chunk (16 or 32)
+    static constexpr int NS = NS_;                           // chunk buffers: NS - 1 chunks of loads in flight
     static constexpr int ROW_BYTES = 1024;                   // one token row of a panel: 16 blocks x 32 x 2 B
-    static constexpr int PANEL_BYTES = TC * ROW_BYTES;       // 32 KB
+    static constexpr int PANEL_BYTES = TC * ROW_BYTES;
     static constexpr int STAGE_BYTES = 2 * PANEL_BYTES;      // G panel, then X panel
     static constexpr int LIST_MAX = SR * SC;
     static constexpr int QMAX = QW * NW;
-    static constexpr int LDS_BYTES = 2 * STAGE_BYTES + LIST_MAX * 4 + LIST_MAX * 2 + (2 * SR + 4) * 4;
+    static constexpr int LDS_BYTES = NS * STAGE_BYTES + LIST_MAX * 4 + LIST_MAX * 2 + (2 * SR + SC / 2 + 4) * 4;
     static constexpr int ROWS_PER_WAVE = TC / NW;            // token rows of each panel a wave copies per chunk
+    static_assert(TC_ == 16 || TC_ == 32, "one or two 16-token matrix steps per chunk");
+    static_assert(NS_ >= 2 && NS_ <= 4, "chunk buffers");
 };
 
-template <int QW>
+template <int QW, int TC_, int NS_>
 __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
-    using C = SddBf16Cfg<QW>;
+    using C = SddBf16Cfg<QW, TC_, NS_>;
+    constexpr int NS = C::NS;
     constexpr int SR = C::SR, SC = C::SC, NW = C::NW, TC = C::TC;
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-    int* s_blk = reinterpret_cast<int*>(smem + 2 * C::STAGE_BYTES);                  // [LIST_MAX] data block
+    int* s_blk = reinterpret_cast<int*>(smem + NS * C::STAGE_BYTES);                  // [LIST_MAX] data block
     unsigned short* s_pos = reinterpret_cast<unsigned short*>(s_blk + C::LIST_MAX);  // [LIST_MAX] (rl << 8) | cl
     int* s_rowoff = reinterpret_cast<int*>(s_pos + C::LIST_MAX);                     // [SR + 1]
     const unsigned lds0 = (unsigned)(uintptr_t)smem;
@@ -59,24 +66,128 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
     const int lrow = lane & 31;
     const int h = lane >> 5;
 
-    // ---- list the blocks of the rectangle, row-major ----
+#ifdef PBS_EXP_TIMING
+    const bool prof_on = (wg == 100) && (lane == 0) && (wave == 0);
+    const int prof_base = 0;
+#endif
+    PBS_T(0);
+    // ---- which rows and columns of W this rectangle covers, and the list of its blocks (row-major) ----
+    // Rows: the band's 16 block rows (sdd_band_rows).  Columns: normally the band's columns c0 .. c0+15.
+    // When the band's entries fit in LDS the columns of the band are instead dealt to the band's
+    // rectangles by block count, in units of two adjacent columns (one 128-byte piece of an X row):
+    // the units are ranked by their number of blocks in this band and handed out in serpentine order.
+    // Rectangles of one band then hold the same number of blocks to within a few, instead of
+    // 64 +- 7 at density 0.25, and the kernel no longer waits for its fullest rectangle.
     int* s_rowid = s_rowoff + SR + 2;   // [SR] block row of W in each place of this rectangle's band, or -1
-    int my_lo = 0, my_n = 0;
-    sdd_band_rows(a.ptr, nblk_r, a.tiles_r, tile / a.tiles_c, SR, s_rowid, reinterpret_cast<int*>(smem), tid, C::NT);
+    int* s_gu = s_rowid + SR;           // [SC / 2] column unit in each place of this rectangle, or -1
+    const int band = tile / a.tiles_c, grp = tile % a.tiles_c;
+    const int nblk_c = a.K / 32;
+    const int nunits = (nblk_c + 1) / 2;
+    sdd_band_rows(a.ptr, nblk_r, a.tiles_r, band, SR, s_rowid, reinterpret_cast<int*>(smem), tid, C::NT);
+    // scratch in the (not yet used) chunk buffers
+    constexpr int EMAX = 8192, UMAX = 1024;
+    int* s_lo = reinterpret_cast<int*>(smem);   // [SR] first entry of each row
+    int* s_rs = s_lo + SR;                      // [SR + 1] start of each row's entries in the cached arrays
+    int* s_ecol = s_rs + SR + 1;                // [EMAX] block column of each cached entry
+    int* s_eblk = s_ecol + EMAX;                // [EMAX] data block of each cached entry
+    int* s_cnt = s_eblk + EMAX;                 // [UMAX] blocks of the band per column unit
+    int* s_ug = s_cnt + UMAX;                   // [UMAX] rectangle * 8 + place of each column unit
+    static_assert((2 * SR + 1 + 2 * EMAX + 2 * UMAX) * 4 <= NS * C::STAGE_BYTES, "scratch fits in the chunk buffers");
+    __syncthreads();
     if (tid < SR) {
         const int r = s_rowid[tid];
-        if (r >= 0) {
-            const int lo = a.ptr[r], hi = a.ptr[r + 1];
-            int l = lo, u = hi;
-            while (l < u) {   // rows are sorted by block column: first entry with column >= c0
-                const int mid = (l + u) >> 1;
-                if (a.idx[2 * mid] < c0) l = mid + 1; else u = mid;
-            }
-            my_lo = l;
-            while (l < hi && a.idx[2 * l] < c0 + SC) ++l;
-            my_n = l - my_lo;
+        const int lo = r >= 0 ? a.ptr[r] : 0, hi = r >= 0 ? a.ptr[r + 1] : 0;
+        s_lo[tid] = lo;
+        s_rs[tid + 1] = hi - lo;
+    }
+    if (tid < SC / 2) s_gu[tid] = -1;
+    __syncthreads();
+    if (tid == 0) {
+        int run = 0;
+        s_rs[0] = 0;
+        for (int i = 0; i < SR; ++i) {
+            run += s_rs[i + 1];
+            s_rs[i + 1] = run;
         }
-        s_rowoff[tid] = my_n;
+    }
+    __syncthreads();
+    const int nent = s_rs[SR];
+    const bool cached = nent <= EMAX;
+    const bool dealt = cached && nunits <= UMAX && a.tiles_c >= 2;
+    int my_lo = 0, my_n = 0;
+    if (cached) {
+        for (int r = 0; r < SR; ++r) {
+            const int lo = s_lo[r], off = s_rs[r], n = s_rs[r + 1] - off;
+            for (int i = tid; i < n; i += C::NT) {
+                const int2 e = *reinterpret_cast<const int2*>(a.idx + 2 * (size_t)(lo + i));
+                s_ecol[off + i] = e.x;
+                s_eblk[off + i] = e.y;
+            }
+        }
+        if (dealt)
+            for (int u = tid; u < nunits; u += C::NT) s_cnt[u] = 0;
+        __syncthreads();
+        if (dealt) {
+            for (int i = tid; i < nent; i += C::NT) {
+                const int c = s_ecol[i];
+                if (c >= 0 && c < nblk_c) atomicAdd(&s_cnt[c >> 1], 1);
+            }
+            __syncthreads();
+            for (int u = tid; u < nunits; u += C::NT) {
+                const int n = s_cnt[u];
+                int rank = 0;
+                for (int o = 0; o < nunits; ++o) {
+                    const int m = s_cnt[o];
+                    rank += (m > n || (m == n && o < u)) ? 1 : 0;
+                }
+                const int place = rank / a.tiles_c;   // < SC / 2: there are at most 8 units per rectangle
+                int gsel = rank % a.tiles_c;
+                if (place & 1) gsel = a.tiles_c - 1 - gsel;
+                s_ug[u] = gsel * (SC / 2) + place;
+                if (gsel == grp) s_gu[place] = u;
+            }
+        } else if (tid < SC / 2) {
+            const int u = grp * (SC / 2) + tid;
+            s_gu[tid] = u < nunits ? u : -1;
+        }
+        __syncthreads();
+        // rows 2*wave and 2*wave + 1: first count this rectangle's blocks, then (below) place them
+        auto mine_of = [&](int c) -> int {   // place (0..15) of block column c in this rectangle, or -1
+            if (c < 0 || c >= nblk_c) return -1;
+            const int ug = dealt ? s_ug[c >> 1] : (c >> 1);
+            return (ug / (SC / 2)) == grp ? (ug % (SC / 2)) * 2 + (c & 1) : -1;
+        };
+#pragma unroll
+        for (int rr = 0; rr < SR / NW; ++rr) {
+            const int r = wave * (SR / NW) + rr;
+            const int off = s_rs[r], n = s_rs[r + 1] - off;
+            int cnt = 0;
+            for (int b0 = 0; b0 < n; b0 += 64) {
+                const bool m = (b0 + lane < n) && mine_of(s_ecol[off + b0 + lane]) >= 0;
+                cnt += __popcll(__ballot(m));
+            }
+            if (lane == 0) s_rowoff[r] = cnt;
+        }
+    } else {
+        if (tid < SC / 2) {
+            const int u = grp * (SC / 2) + tid;
+            s_gu[tid] = u < nunits ? u : -1;
+        }
+        if (tid < SR) {
+            const int r = s_rowid[tid];
+            if (r >= 0) {
+                const int lo = a.ptr[r], hi = a.ptr[r + 1];
+                int l = lo, u = hi;
+                while (l < u) {   // rows are sorted by block column: first entry with column >= c0
+                    const int mid = (l + u) >> 1;
+                    if (a.idx[2 * mid] < c0) l = mid + 1; else u = mid;
+                }
+                my_lo = l;
+                while (l < hi && a.idx[2 * l] < c0 + SC) ++l;
+                my_n = l - my_lo;
+            }
+            s_rowoff[tid] = my_n;
+        }
     }
     __syncthreads();
     if (tid == 0) {
@@ -89,7 +200,31 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
         s_rowoff[SR] = run;
     }
     __syncthreads();
-    if (tid < SR) {
+    if (cached) {
+        auto mine_of = [&](int c) -> int {
+            if (c < 0 || c >= nblk_c) return -1;
+            const int ug = dealt ? s_ug[c >> 1] : (c >> 1);
+            return (ug / (SC / 2)) == grp ? (ug % (SC / 2)) * 2 + (c & 1) : -1;
+        };
+#pragma unroll
+        for (int rr = 0; rr < SR / NW; ++rr) {
+            const int r = wave * (SR / NW) + rr;
+            const int off = s_rs[r], n = s_rs[r + 1] - off;
+            int run = s_rowoff[r];
+            for (int b0 = 0; b0 < n; b0 += 64) {
+                const int cl = (b0 + lane < n) ? mine_of(s_ecol[off + b0 + lane]) : -1;
+                const unsigned long long bal = __ballot(cl >= 0);
+                if (cl >= 0) {
+                    const int at = run + __popcll(bal & ((1ull << lane) - 1ull));
+                    int b = s_eblk[off + b0 + lane];
+                    if (b < 0 || b >= a.nnz) b = -1;
+                    s_blk[at] = b;
+                    s_pos[at] = (unsigned short)((r << 8) | cl);
+                }
+                run += __popcll(bal);
+            }
+        }
+    } else if (tid < SR) {
         const int off = s_rowoff[tid];
         for (int i = 0; i < my_n; ++i) {
             const int c = a.idx[2 * (my_lo + i)];
@@ -102,6 +237,7 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
     __syncthreads();
     const int nq = __builtin_amdgcn_readfirstlane(s_rowoff[SR]);
     if (nq == 0) return;
+    PBS_T(1);
 
     const int t_begin = sp * a.tokens_per_split;
     int t_end = t_begin + a.tokens_per_split;
@@ -112,20 +248,25 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
     //      chunk swizzle of those rows is the same ((wave & 3) << 2) ----
     const unsigned char* G = static_cast<const unsigned char*>(a.g);
     const unsigned char* X = static_cast<const unsigned char*>(a.x);
-    const int x_valid = (a.K - c0 * 32) * 2;
     const int pc = lane ^ ((wave & 3) << 2);   // panel chunk fetched by this lane
     // G: the 64 bytes of place pc / 4 of the band come from that place's block row (a place without a
     // row fetches any valid address; nothing reads it)
     const int g_rid = s_rowid[pc >> 2];
     const unsigned g_voff = g_rid >= 0 ? (unsigned)(g_rid * 64 + (pc & 3) * 16) : 0u;
-    const unsigned x_voff = (pc * 16 < x_valid) ? pc * 16 : 0;
+    // X: the 64 bytes of place pc / 4 come from that place's block column (two adjacent columns per unit)
+    const int x_unit = s_gu[pc >> 3];
+    const int x_cid = x_unit >= 0 ? x_unit * 2 + ((pc >> 2) & 1) : -1;
+    const unsigned x_voff = (x_cid >= 0 && x_cid < nblk_c) ? (unsigned)(x_cid * 64 + (pc & 3) * 16) : 0u;
     const size_t g_row_bytes = (size_t)a.N * 2, x_row_bytes = (size_t)a.K * 2;
     const unsigned char* g_col = G;
-    const unsigned char* x_col = X + (size_t)c0 * 64;
+    const unsigned char* x_col = X;
 
-    auto issue_chunk = [&](int ci) {
+    // returns the number of DMA instructions issued (wave-uniform)
+    auto issue_chunk = [&](int ci) -> int {
         const int t0 = t_begin + ci * TC;
-        const unsigned stage = lds0 + (ci & 1) * C::STAGE_BYTES;
+        const int buf = ci % NS;
+        const unsigned stage = lds0 + buf * C::STAGE_BYTES;
+        int n = 0;
 #pragma unroll
         for (int k = 0; k < C::ROWS_PER_WAVE; ++k) {
             const int tl = wave + k * NW;
@@ -133,13 +274,15 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
             if (t < t_end) {
                 dma16(stage + tl * C::ROW_BYTES, uniform_ptr(g_col + (size_t)t * g_row_bytes), g_voff);
                 dma16(stage + C::PANEL_BYTES + tl * C::ROW_BYTES, uniform_ptr(x_col + (size_t)t * x_row_bytes), x_voff);
+                n += 2;
             } else {
                 // tokens past the end contribute nothing
-                unsigned char* p = smem + (ci & 1) * C::STAGE_BYTES + tl * C::ROW_BYTES + lane * 16;
+                unsigned char* p = smem + buf * C::STAGE_BYTES + tl * C::ROW_BYTES + lane * 16;
                 *reinterpret_cast<uint4*>(p) = make_uint4(0, 0, 0, 0);
                 *reinterpret_cast<uint4*>(p + C::PANEL_BYTES) = make_uint4(0, 0, 0, 0);
             }
         }
+        return n;
     };
 
     // ---- per-lane part of the fragment addresses ----
@@ -182,17 +325,18 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[q][v] = 0.f;
 
-        auto load_frag = [&](uint4 (&f)[2], const unsigned char* p) {
+        constexpr int NU = TC / 16;   // 16-token matrix steps per chunk
+        auto load_frag = [&](uint4 (&f)[NU], const unsigned char* p) {
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
+            for (int u = 0; u < NU; ++u) {
                 const uint2 lo = tr16_b64(p + (16 * u) * C::ROW_BYTES);
                 const uint2 hi = tr16_b64(p + (16 * u + 4) * C::ROW_BYTES);
                 f[u] = make_uint4(lo.x, lo.y, hi.x, hi.y);
             }
         };
         auto compute_chunk = [&](int ci) {
-            const unsigned char* stage = smem + (ci & 1) * C::STAGE_BYTES;
-            uint4 fb[2];
+            const unsigned char* stage = smem + (ci % NS) * C::STAGE_BYTES;
+            uint4 fb[NU];
             int cur_rl = -1;
 #pragma unroll
             for (int q = 0; q < QW; ++q) {
@@ -201,23 +345,43 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
                         load_frag(fb, stage + b_off[q]);
                         cur_rl = rl_of[q];
                     }
-                    uint4 fa[2];
+                    uint4 fa[NU];
                     load_frag(fa, stage + a_off[q]);
-                    Elem<bf16_t>::mma(acc[q], fa, fb);
+#pragma unroll
+                    for (int u = 0; u < NU; ++u)
+                        acc[q] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa[u]),
+                                                                         __builtin_bit_cast(bf16x8, fb[u]), acc[q], 0, 0, 0);
                 }
             }
         };
 
         if (nchunks > 0) {
-            issue_chunk(0);
+            // DMA counts of the chunks in flight, oldest (the one computed next) first
+            int pend[NS];
+#pragma unroll
+            for (int k = 0; k < NS; ++k) pend[k] = 0;
+#pragma unroll
+            for (int k = 0; k < NS - 1; ++k)
+                if (k < nchunks) pend[k] = issue_chunk(k);
             for (int ci = 0; ci < nchunks; ++ci) {
-                // only chunk ci is in flight here; the other buffer was read by chunk ci-1
-                drain_barrier();
-                if (ci + 1 < nchunks) issue_chunk(ci + 1);
+                PBS_T(8 + 4 * ci + 0);
+                int later = 0;
+#pragma unroll
+                for (int k = 1; k < NS; ++k) later += pend[k];
+                // chunk ci has landed for every wave, and every wave is done reading chunk ci - 1
+                wait_dma_and_barrier(later);
+                PBS_T(8 + 4 * ci + 1);
+#pragma unroll
+                for (int k = 0; k + 1 < NS; ++k) pend[k] = pend[k + 1];
+                pend[NS - 1] = 0;
+                if (ci + NS - 1 < nchunks) pend[NS - 2] = issue_chunk(ci + NS - 1);   // into the buffer of chunk ci - 1
+                PBS_T(8 + 4 * ci + 2);
                 compute_chunk(ci);
+                PBS_T(8 + 4 * ci + 3);
             }
-            lds_barrier();   // the next pass refills buffer 0
+            lds_barrier();   // the next pass refills the buffers
         }
+        PBS_T(2);
 
         // ---- store: result row j (X feature), column i (G feature) ----
 #pragma unroll
@@ -231,6 +395,7 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
                 }
             }
         }
+        PBS_T(3);
     }
 }
 
