@@ -140,7 +140,7 @@ static int dispatch_dds(const DdsArgs& g, hipStream_t stream) {
 // fp32: 8 x 8 rectangles, 16-token chunks staged through registers; bf16: 16 x 16 rectangles,
 // 32-token chunks by DMA.
 struct SddShapeF32 {
-    static constexpr int SR = 8, SC = 8, QW = 8, NW = 4, TC = 16;
+    static constexpr int SR = 8, SC = 8, QW = 8, NW = 8, TC = 16;
 };
 #ifndef PBS_EXP_SDD_TC
 #define PBS_EXP_SDD_TC 32
