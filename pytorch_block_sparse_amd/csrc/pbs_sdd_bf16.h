@@ -262,26 +262,27 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
     const unsigned char* x_col = X;
 
     // returns the number of DMA instructions issued (wave-uniform)
-    auto issue_chunk = [&](int ci) -> int {
-        const int t0 = t_begin + ci * TC;
+    // token row number k of this wave's ROWS_PER_WAVE, both panels, of chunk ci; returns the DMA count
+    auto issue_row = [&](int ci, int k) -> int {
         const int buf = ci % NS;
-        const unsigned stage = lds0 + buf * C::STAGE_BYTES;
+        const int tl = wave + k * NW;
+        const int t = t_begin + ci * TC + tl;
+        if (t < t_end) {
+            const unsigned stage = lds0 + buf * C::STAGE_BYTES + tl * C::ROW_BYTES;
+            dma16(stage, uniform_ptr(g_col + (size_t)t * g_row_bytes), g_voff);
+            dma16(stage + C::PANEL_BYTES, uniform_ptr(x_col + (size_t)t * x_row_bytes), x_voff);
+            return 2;
+        }
+        // tokens past the end contribute nothing
+        unsigned char* p = smem + buf * C::STAGE_BYTES + tl * C::ROW_BYTES + lane * 16;
+        *reinterpret_cast<uint4*>(p) = make_uint4(0, 0, 0, 0);
+        *reinterpret_cast<uint4*>(p + C::PANEL_BYTES) = make_uint4(0, 0, 0, 0);
+        return 0;
+    };
+    auto issue_chunk = [&](int ci) -> int {
         int n = 0;
 #pragma unroll
-        for (int k = 0; k < C::ROWS_PER_WAVE; ++k) {
-            const int tl = wave + k * NW;
-            const int t = t0 + tl;
-            if (t < t_end) {
-                dma16(stage + tl * C::ROW_BYTES, uniform_ptr(g_col + (size_t)t * g_row_bytes), g_voff);
-                dma16(stage + C::PANEL_BYTES + tl * C::ROW_BYTES, uniform_ptr(x_col + (size_t)t * x_row_bytes), x_voff);
-                n += 2;
-            } else {
-                // tokens past the end contribute nothing
-                unsigned char* p = smem + buf * C::STAGE_BYTES + tl * C::ROW_BYTES + lane * 16;
-                *reinterpret_cast<uint4*>(p) = make_uint4(0, 0, 0, 0);
-                *reinterpret_cast<uint4*>(p + C::PANEL_BYTES) = make_uint4(0, 0, 0, 0);
-            }
-        }
+        for (int k = 0; k < C::ROWS_PER_WAVE; ++k) n += issue_row(ci, k);
         return n;
     };
 
