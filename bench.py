@@ -156,7 +156,17 @@ def main():
     dom = max(per_kernel, key=per_kernel.get)
     achieved = flops_gemm / (per_kernel[dom] * 1e-3) / 1e12
     sdd = "sdd_bf16_kernel" if dname == "bf16" else "sdd_kernel"
-    kernel_names = {"fwd": "dds_kernel<TRANS=0>", "dx": "dds_kernel<TRANS=1>", "dw": sdd + " (+ sdd_reduce_kernel)"}
+
+    def dds_name(n, k, trans):
+        # the library picks the wide-tile kernel for bf16 when there are at least 256 tiles of 128 tokens x 512 columns
+        wide = dname == "bf16" and k % 64 == 0 and ((tokens + 127) // 128) * ((n // 32 + 15) // 16) >= 256
+        return ("dds16_kernel" if wide else "dds_kernel") + f"<TRANS={trans}>"
+
+    kernel_names = {
+        "fwd": dds_name(w.out_features, w.in_features, 0),
+        "dx": dds_name(w.in_features, w.out_features, 1),
+        "dw": sdd + " (+ sdd_reduce_kernel)",
+    }
     traffic = MEASURED_TRAFFIC.get((w.name, tokens), {}).get(dom)
 
     out = {

@@ -293,7 +293,8 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
         // minimum over the compute waves of (steps done, entries done): lanes 0..7 read lane 0's pair of
         // each wave, three row shifts bring the minimum to lane 7
         auto consumers_done = [&](int& steps, int& entries) {
-            const volatile int* pw = s_done + (lane & 7) * 64;
+            // every lane of a compute wave writes its own copy; reading copy w of wave w puts the 8 words on 8 banks
+            const volatile int* pw = s_done + (lane & 7) * 64 + (lane & 7);
             int a = pw[0], b = pw[NW * 64];
 #define PBS_MIN_SHR(SH)                                                                  \
     {                                                                                    \
@@ -446,7 +447,7 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
     // Steps whose operands have arrived from every copy wave.  The words hold the count modulo 256 and
     // are never more than the ring depth away from u, so the signed 8-bit difference is exact.
     auto producers_landed = [&](int u) -> int {
-        const int v = *(const volatile int*)(s_landed + (lane & 3) * 64);
+        const int v = *(const volatile int*)(s_landed + (lane & 3) * 64 + (lane & 3));   // copy c of wave c: 4 banks
         int m = 127;
 #pragma unroll
         for (int c = 0; c < NP; ++c) {
