@@ -104,11 +104,104 @@ def cpu_baseline(w, sample_tokens):
     }
 
 
+ROBERTA_WORKLOAD = "c5_roberta_base_mlm_fp32"
+
+
+def run_roberta(args):
+    """One MLM training step (forward + backward + AdamW, fp32) of a 12-layer RoBERTa-base-shaped encoder
+    with random weights, batch 32 x 512 random token ids, once with dense linear layers and once with
+    attention.output.dense, intermediate.dense and output.dense of every layer patched to block-sparse
+    layers of density 0.5 (the reference's tests/test_integration.py:66-113 procedure at full size)."""
+    import torch
+    from transformers import RobertaConfig, RobertaForMaskedLM
+
+    from pytorch_block_sparse_amd import BlockSparseLinear, BlockSparseModelPatcher, native
+
+    native.load()
+    dev = torch.device("cuda:0")
+    batch, seq = 32, 512
+    cfg = RobertaConfig(vocab_size=50265, hidden_size=768, num_hidden_layers=12, num_attention_heads=12,
+                        intermediate_size=3072, max_position_embeddings=seq + 2,
+                        hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0)
+    g = torch.Generator().manual_seed(0)
+    ids = torch.randint(0, cfg.vocab_size, (batch, seq), generator=g)
+    labels = ids.clone()
+    labels[torch.rand((batch, seq), generator=g) >= 0.15] = -100   # 15 % of the positions are predicted
+    ids, labels = ids.to(dev), labels.to(dev)
+
+    def build(sparse):
+        torch.manual_seed(1)
+        model = RobertaForMaskedLM(cfg)
+        n_dense = sum(p.numel() for p in model.parameters())
+        model = model.to(dev)
+        n_layers = 0
+        if sparse:
+            mp = BlockSparseModelPatcher()
+            for pat in (r"roberta\.encoder\.layer\.[0-9]+\.attention\.output\.dense",
+                        r"roberta\.encoder\.layer\.[0-9]+\.intermediate\.dense",
+                        r"roberta\.encoder\.layer\.[0-9]+\.output\.dense"):
+                mp.add_pattern(pat, {"density": 0.5})
+            mp.patch_model(model)
+            n_layers = sum(isinstance(m, BlockSparseLinear) for m in model.modules())
+        return model, n_dense, sum(p.numel() for p in model.parameters()), n_layers
+
+    def time_model(model):
+        opt = torch.optim.AdamW(model.parameters(), lr=1e-4)
+
+        def one():
+            loss = model(input_ids=ids, labels=labels).loss
+            loss.backward()
+            opt.step()
+            opt.zero_grad(set_to_none=True)
+            return loss
+
+        for _ in range(args.warmup):
+            one()
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(args.steps):
+            loss = one()
+        end.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(end) / args.steps, float(loss)
+
+    model, n_dense, _, _ = build(False)
+    ms_dense, loss_dense = time_model(model)
+    del model
+    torch.cuda.empty_cache()
+    model, _, n_sparse, n_layers = build(True)
+    ms_sparse, loss_sparse = time_model(model)
+    tokens = batch * seq
+    print(json.dumps({
+        "metric": "MLM training step of a RoBERTa-base-shaped encoder, 36 linear layers block-sparse at density 0.5",
+        "value": tokens / (ms_sparse * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_sparse,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": ROBERTA_WORKLOAD, "layers": 12, "hidden": 768, "ffn": 3072, "vocab": 50265,
+                   "batch": batch, "seq_len": seq, "density": 0.5, "patched_layers": n_layers},
+        "dense_model": {"ms_per_step": ms_dense, "parameters": n_dense, "loss": loss_dense},
+        "sparse_model": {"ms_per_step": ms_sparse, "parameters": n_sparse, "loss": loss_sparse},
+        "speedup_sparse_vs_dense": ms_dense / ms_sparse,
+    }))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only; --gpus must be 1", file=sys.stderr)
         sys.exit(2)
+    if args.workload == ROBERTA_WORKLOAD:
+        run_roberta(args)
+        return
     import torch
 
     from pytorch_block_sparse_amd import BlockSparseMatrix, native, workloads
@@ -146,8 +239,25 @@ def main():
         for f in kernels.values():
             f()
 
-    ms_step = time_gpu(step, args.steps, args.warmup)
-    per_kernel = {k: time_gpu(f, args.steps, min(args.warmup, 3)) for k, f in kernels.items()}
+    # The timed region is exactly `steps` steps.  Inside it an event is recorded after every kernel, so
+    # that the per-kernel durations are those of the launches of the timed steps themselves (the same
+    # launches a rocprofv3 kernel trace of this command averages), not of a kernel repeated on its own.
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    names = list(kernels)
+    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(len(names) + 1)] for _ in range(args.steps)]
+    for i in range(args.steps):
+        marks[i][0].record()
+        for j, kname in enumerate(names):
+            kernels[kname]()
+            marks[i][j + 1].record()
+    torch.cuda.synchronize()
+    ms_step = marks[0][0].elapsed_time(marks[-1][-1]) / args.steps
+    per_kernel = {
+        kname: sum(marks[i][j].elapsed_time(marks[i][j + 1]) for i in range(args.steps)) / args.steps
+        for j, kname in enumerate(names)
+    }
 
     dname = "bf16" if w.dtype == torch.bfloat16 else "f32"
     flops_gemm = 2.0 * tokens * w.nnz * 1024
