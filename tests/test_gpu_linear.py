@@ -186,3 +186,37 @@ def test_patched_model_trains_and_sparse_optimizer(cuda, capsys):
             y = model.mid.weight.reverse_matmul(x @ model.inp.weight.t(), True)
             assert torch.allclose(y, (x @ model.inp.weight.t()) @ d.t(), rtol=1e-4, atol=1e-4)
     assert all(np.isfinite(losses)) and losses[-1] < losses[0]
+
+
+def test_roberta_patched_at_full_density_keeps_outputs(cuda):
+    """reference tests/test_integration.py:66-113 (test1), two encoder layers instead of six: patching the
+    feed-forward linears of a RoBERTa masked-LM model at density 1.0 keeps parameter count and logits;
+    at density 0.5 the patched weights halve."""
+    transformers = pytest.importorskip("transformers")
+    torch.manual_seed(3)
+    np.random.seed(3)
+    config = transformers.RobertaConfig(vocab_size=52_000, max_position_embeddings=514, num_attention_heads=12,
+                                        num_hidden_layers=2, type_vocab_size=1)
+    patterns = [r"roberta\.encoder\.layer\.[0-9]+.intermediate\.dense", r"roberta\.encoder\.layer\.[0-9]+.output\.dense"]
+
+    def patch(model, density):
+        mp = BlockSparseModelPatcher()
+        for p in patterns:
+            mp.add_pattern(p, {"density": density})
+        mp.patch_model(model)
+        return model
+
+    model = transformers.RobertaForMaskedLM(config=config).to(cuda).eval()
+    n0 = model.num_parameters()
+    input_ids = torch.tensor([[4, 5, 6, 7] * 8], device=cuda)
+    with torch.no_grad():
+        out0 = model(input_ids)[0]
+        patch(model, 1.0)
+        out1 = model(input_ids)[0]
+    assert sum(isinstance(m, BlockSparseLinear) for m in model.modules()) == 4
+    assert model.num_parameters() == n0
+    assert torch.isclose(out0, out1, atol=1e-3).all()
+    model2 = patch(transformers.RobertaForMaskedLM(config=config).to(cuda).eval(), 0.5)
+    with torch.no_grad():
+        assert torch.isfinite(model2(input_ids)[0]).all()
+    assert model2.num_parameters() == n0 - 4 * (768 * 3072 // 2)
