@@ -141,7 +141,7 @@ struct D16Cfg {
     // 8 compute waves = (4 / TM) token slices of TM * 32 tokens x (2 * TM) column groups of NBW = 8 / TM block
     // columns; wave w has slice w % (4 / TM), so the waves that share a SIMD (w, w + 4) share their slice
     static constexpr int NW = 8, NT = (NW + NP) * 64, BM = D16_BM, TM = TM_, NBW = 8 / TM_, NSL = 4 / TM_;
-    static_assert(TM_ == 1 || TM_ == 2, "token sub-slices per wave");
+    static_assert(TM_ == 1 || TM_ == 2 || TM_ == 4, "token sub-slices per wave");
     static constexpr int ROWB = 128;                          // one panel row: 64 k values
     static constexpr int PANEL_BYTES = BM * ROWB;             // 16 KB per step
     static constexpr int A_PER_WAVE = PANEL_BYTES / 1024 / NP;
@@ -320,12 +320,19 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
             const int cnt = __popc((unsigned)__builtin_amdgcn_readlane(vrec, D16_F_MASK));
             const int e0 = jn * ne + __builtin_amdgcn_readlane(vrec, D16_F_CUM);
             const int end_t = e0 + cnt;
+            bool free_now = false;
             for (int spin = 0; spin < C::SPIN_LIMIT; ++spin) {
                 int steps, entries;
                 consumers_done(steps, entries);
-                if (steps >= t - RS + 1 && end_t - entries <= RB) break;
+                if (steps >= t - RS + 1 && end_t - entries <= RB) {
+                    free_now = true;
+                    break;
+                }
                 __builtin_amdgcn_s_sleep(1);
             }
+            // Cannot happen unless the protocol is broken: stop feeding rather than overwrite operands in
+            // use; the compute waves then run into their own limit and mark the result (see there).
+            if (!free_now) break;
             wait_dma(63 - C::MAX_STEP_DMA - 1);   // the counter of outstanding loads has 6 bits
             asm volatile("" ::: "memory");
             PBS_T(8 + 4 * t + 1);
@@ -411,31 +418,34 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
         asm volatile("" : "+v"(l));
         const int er = l & 31, eh = l >> 5;
         const int m0 = (p + j * g.wg_per_group) * C::BM;
+        constexpr int CW = NBW < 4 ? NBW : 4;          // block columns staged at a time
+        constexpr int CHUNKS = CW * 4;                 // 16-byte pieces per staged row
+        constexpr int ROWS_PER_READ = 64 / CHUNKS;     // staged rows one wave-wide read covers
         bf16_t* st_w = stage + (4 * eh) * C::STAGE_ROW + er;                    // + vv rows, + jc*32
-        const int rd_r = l >> 4, rd_c = (l & 15) * 8;
-        const bf16_t* st_r = stage + rd_r * C::STAGE_ROW + rd_c;                // + 4 rows for the second read
+        const int rd_r = l / CHUNKS, rd_c = (l % CHUNKS) * 8;
+        const bf16_t* st_r = stage + rd_r * C::STAGE_ROW + rd_c;                // + ROWS_PER_READ rows per further read
 #pragma unroll
-        for (int cg = 0; cg < NBW / 4; ++cg) {   // 4 block columns (128 result columns) at a time
-            float bv[4];
+        for (int cg = 0; cg < NBW / CW; ++cg) {   // CW block columns at a time
+            float bv[CW];
 #pragma unroll
-            for (int jc = 0; jc < 4; ++jc) {
-                const int col = col0 + (cg * 4 + jc) * 32 + er;
+            for (int jc = 0; jc < CW; ++jc) {
+                const int col = col0 + (cg * CW + jc) * 32 + er;
                 bv[jc] = (bias && col < g.N) ? E::to_f32(bias[col]) : 0.f;
             }
-            const int col = col0 + cg * 128 + rd_c;
+            const int col = col0 + cg * CW * 32 + rd_c;
 #pragma unroll
             for (int t = 0; t < TM; ++t) {
 #pragma unroll
                 for (int gq = 0; gq < 4; ++gq) {
 #pragma unroll
-                    for (int jc = 0; jc < 4; ++jc)
+                    for (int jc = 0; jc < CW; ++jc)
 #pragma unroll
                         for (int vv = 0; vv < 4; ++vv)
-                            st_w[vv * C::STAGE_ROW + jc * 32] = E::from_f32(acc[t][cg * 4 + jc][4 * gq + vv] + bv[jc]);
+                            st_w[vv * C::STAGE_ROW + jc * 32] = E::from_f32(acc[t][cg * CW + jc][4 * gq + vv] + bv[jc]);
 #pragma unroll
-                    for (int pp = 0; pp < 2; ++pp) {
-                        const uint4 val = *reinterpret_cast<const uint4*>(st_r + pp * 4 * C::STAGE_ROW);
-                        const int row = m0 + (ms * TM + t) * 32 + gq * 8 + pp * 4 + rd_r;
+                    for (int pp = 0; pp < 8 / ROWS_PER_READ; ++pp) {
+                        const uint4 val = *reinterpret_cast<const uint4*>(st_r + pp * ROWS_PER_READ * C::STAGE_ROW);
+                        const int row = m0 + (ms * TM + t) * 32 + gq * 8 + pp * ROWS_PER_READ + rd_r;
                         if (row < g.M && col < g.N) *reinterpret_cast<uint4*>(out + (size_t)row * g.N + col) = val;
                     }
                 }
@@ -467,6 +477,14 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
                     landed = producers_landed(u);
                     if (landed > u) break;
                     __builtin_amdgcn_s_sleep(1);
+                }
+                // Operands that never arrive mean a broken protocol, not a slow machine (a wave that is
+                // not running does not count polls).  Make the failure visible: the tile becomes NaN.
+                if (landed <= u) {
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int jc = 0; jc < NBW; ++jc) acc[i][jc][0] = __builtin_nanf("");
                 }
             }
             asm volatile("" ::: "memory");   // operand reads stay behind the poll
