@@ -155,7 +155,7 @@ struct D16Cfg {
     // progress words: done steps [NW][64] then done entries [NW][64] (every lane of a compute wave writes
     // its own copy, lane 0's is read), then landed [NP][64] (the progress DMA writes one copy per lane)
     static constexpr int DONE_BYTES = NW * 64 * 8;
-    static constexpr int FLAG_BYTES = DONE_BYTES + NP * 256;   // landed[c]: 64 copies of one word per copy wave
+    static constexpr int FLAG_BYTES = DONE_BYTES + NP * 256 + 256;   // landed[c]: 64 copies of one word per copy wave; failure word
     static constexpr int FLAG_OFF = A_RING_BYTES + B_RING_BYTES + STAGE_BYTES;
     static constexpr int WORK_BYTES = FLAG_OFF + FLAG_BYTES;   // + the plan records
     static constexpr int SPIN_LIMIT = 1 << 20;                // polls before a wave gives up waiting
@@ -197,6 +197,7 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
     // ---- this group's plan records -> LDS; progress words start at zero ----
     int* const s_done = reinterpret_cast<int*>(smem + C::FLAG_OFF);                     // [2][NW][64]
     int* const s_landed = reinterpret_cast<int*>(smem + C::FLAG_OFF + C::DONE_BYTES);   // [NP]
+    int* const s_fail = s_landed + NP * 64;   // set by a copy wave whose wait ran into its bound
     {
         const int4* src = reinterpret_cast<const int4*>(g.plan + (size_t)ng * g.group_ints);
         int4* dst = reinterpret_cast<int4*>(s_plan);
@@ -330,9 +331,8 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
                 }
                 __builtin_amdgcn_s_sleep(1);
             }
-            // Cannot happen unless the protocol is broken: stop feeding rather than overwrite operands in
-            // use; the compute waves then run into their own limit and mark the result (see there).
-            if (!free_now) break;
+            // Cannot happen unless the protocol is broken: say so; the compute waves mark their results.
+            if (!free_now) *(volatile int*)s_fail = 1;
             wait_dma(63 - C::MAX_STEP_DMA - 1);   // the counter of outstanding loads has 6 bits
             asm volatile("" ::: "memory");
             PBS_T(8 + 4 * t + 1);
@@ -398,6 +398,7 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
     const int col0 = (nb0 + quarter * NBW) * 32;   // first result column of this wave
     bf16_t* stage = reinterpret_cast<bf16_t*>(smem + C::A_RING_BYTES + C::B_RING_BYTES + wave * C::STAGE_WAVE_BYTES);
 
+    bool gave_up = false;   // a wait ran into its bound (broken protocol): results are marked NaN
     f32x16 acc[TM][NBW];
     auto zero_acc = [&]() {
 #pragma unroll
@@ -418,6 +419,7 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
         asm volatile("" : "+v"(l));
         const int er = l & 31, eh = l >> 5;
         const int m0 = (p + j * g.wg_per_group) * C::BM;
+        const bool failed = __builtin_amdgcn_readfirstlane(*(const volatile int*)s_fail) != 0;
         constexpr int CW = NBW < 4 ? NBW : 4;          // block columns staged at a time
         constexpr int CHUNKS = CW * 4;                 // 16-byte pieces per staged row
         constexpr int ROWS_PER_READ = 64 / CHUNKS;     // staged rows one wave-wide read covers
@@ -431,6 +433,7 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
             for (int jc = 0; jc < CW; ++jc) {
                 const int col = col0 + (cg * CW + jc) * 32 + er;
                 bv[jc] = (bias && col < g.N) ? E::to_f32(bias[col]) : 0.f;
+                if (gave_up || failed) bv[jc] = __builtin_nanf("");
             }
             const int col = col0 + cg * CW * 32 + rd_c;
 #pragma unroll
@@ -479,13 +482,8 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
                     __builtin_amdgcn_s_sleep(1);
                 }
                 // Operands that never arrive mean a broken protocol, not a slow machine (a wave that is
-                // not running does not count polls).  Make the failure visible: the tile becomes NaN.
-                if (landed <= u) {
-#pragma unroll
-                    for (int i = 0; i < TM; ++i)
-#pragma unroll
-                        for (int jc = 0; jc < NBW; ++jc) acc[i][jc][0] = __builtin_nanf("");
-                }
+                // not running does not count polls).  Make the failure visible: the tiles become NaN.
+                if (landed <= u) gave_up = true;
             }
             asm volatile("" ::: "memory");   // operand reads stay behind the poll
             PBS_T(8 + 4 * u + 1);
