@@ -267,14 +267,11 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
         // Returns the instruction count.
         auto issue_step = [&](unsigned stage, int vrec, int e0, int cnt) -> int {
             int n = 0;
-#ifndef PBS_EXP_NO_A
             const int pair = __builtin_amdgcn_readlane(vrec, D16_F_PAIR);
             const unsigned char* src = uniform_ptr(a_tile + (size_t)pair * C::ROWB);
 #pragma unroll
             for (int q = 0; q < C::A_PER_WAVE; ++q) dma16(stage + q * 1024, src, a_voff[q]);
             n = C::A_PER_WAVE;
-#endif
-#ifndef PBS_EXP_NO_B
 #pragma unroll
             for (int k = 0; k < 2 * D16_NB / NP; ++k) {
                 const int i = dw + k * NP;
@@ -287,7 +284,6 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
                     n += 2;
                 }
             }
-#endif
             return n;
         };
 
@@ -496,11 +492,7 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk) {
                 const unsigned mk = (mask >> (16 * kk)) & 0xffffu;
-#ifdef PBS_EXP_NO_COMPUTE
-                const unsigned mine = 0;
-#else
                 const unsigned mine = (mk >> (NBW * quarter)) & ((1u << NBW) - 1u);
-#endif
                 if (mine == 0) continue;
                 const int e0 = base + (kk ? __popc(mask & 0xffffu) : 0) + __popc(mk & ((1u << (NBW * quarter)) - 1u));
                 // One register index at a time keeps only 12 fragment registers live next to the 128

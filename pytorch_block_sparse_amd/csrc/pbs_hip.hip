@@ -69,10 +69,7 @@ static inline size_t wide_plan_bytes(int n, int k) {
     return (groups * dds16_plan_group_ints(k / 32) + D16_SEQ_INTS) * sizeof(int);
 }
 
-#ifndef PBS_EXP_D16_TM
-#define PBS_EXP_D16_TM 2
-#endif
-constexpr int D16_TM = PBS_EXP_D16_TM, D16_RS = 3, D16_RB = 32, D16_NP = 4;
+constexpr int D16_TM = 2, D16_RS = 3, D16_RB = 32, D16_NP = 4;
 
 // Whether the wide kernel serves this problem: k-pairs need k % 64 == 0, the plan records of a group
 // must fit in LDS beside the rings, and there must be enough tiles to give every CU one.
@@ -142,12 +139,8 @@ static int dispatch_dds(const DdsArgs& g, hipStream_t stream) {
 struct SddShapeF32 {
     static constexpr int SR = 8, SC = 8, QW = 8, NW = 8, TC = 16;
 };
-#ifndef PBS_EXP_SDD_TC
-#define PBS_EXP_SDD_TC 32
-#define PBS_EXP_SDD_NS 2
-#endif
 struct SddShapeBf16 {
-    static constexpr int SR = 16, SC = 16, QW = 10, TC = PBS_EXP_SDD_TC, NS = PBS_EXP_SDD_NS;
+    static constexpr int SR = 16, SC = 16, QW = 10, TC = 32, NS = 2;
 };
 
 struct SddPlan {
