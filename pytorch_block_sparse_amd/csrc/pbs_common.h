@@ -96,6 +96,13 @@ static __device__ __forceinline__ uint2 tr16_b64(const unsigned char* lds_ptr) {
     return __builtin_bit_cast(uint2, v);
 }
 
+// Volatile accesses to LDS words other waves write or poll.  The pointer is cast to the LDS address
+// space explicitly: a volatile access through a generic pointer is compiled to a flat instruction,
+// which takes the long way round through the vector memory path.
+typedef int __attribute__((address_space(3))) lds_int;
+static __device__ __forceinline__ int lds_peek(const int* p) { return *(const volatile lds_int*)p; }
+static __device__ __forceinline__ void lds_poke(int* p, int v) { *(volatile lds_int*)p = v; }
+
 // a wave-uniform pointer, forced into scalar registers
 static __device__ __forceinline__ const unsigned char* uniform_ptr(const unsigned char* p) {
     const uint64_t v = reinterpret_cast<uint64_t>(p);

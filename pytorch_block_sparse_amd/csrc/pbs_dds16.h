@@ -261,6 +261,11 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
                 a_voff[q] = (unsigned)r * (unsigned)a_row_bytes + a_chunk[q];
             }
             a_tile = uniform_ptr(A + (size_t)m0 * a_row_bytes);
+#ifdef PBS_EXP_SAMEA
+            a_tile = A;
+#pragma unroll
+            for (int q = 0; q < C::A_PER_WAVE; ++q) a_voff[q] = (unsigned)a_row[q] * (unsigned)a_row_bytes + a_chunk[q];
+#endif
         };
         // Issue the DMA of global step t (panel buffer `stage`, records in vrec, e0 entries before it).
         // The blocks of a step are dealt to the copy waves by entry number (dw, dw + 4, ...).
@@ -276,7 +281,10 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
             for (int k = 0; k < 2 * D16_NB / NP; ++k) {
                 const int i = dw + k * NP;
                 if (i < cnt) {
-                    const unsigned id = (unsigned)__builtin_amdgcn_readlane(vrec, i);
+                    unsigned id = (unsigned)__builtin_amdgcn_readlane(vrec, i);
+#ifdef PBS_EXP_SAMEW
+                    id &= 63u;
+#endif
                     const unsigned char* bsrc = uniform_ptr(D + ((size_t)id << 11));
                     const unsigned bdst = lds_b + (((unsigned)(e0 + i) & (RB - 1)) << 11);
                     dma16(bdst, bsrc, b_voff[0]);
@@ -291,8 +299,8 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
         // each wave, three row shifts bring the minimum to lane 7
         auto consumers_done = [&](int& steps, int& entries) {
             // every lane of a compute wave writes its own copy; reading copy w of wave w puts the 8 words on 8 banks
-            const volatile int* pw = s_done + (lane & 7) * 64 + (lane & 7);
-            int a = pw[0], b = pw[NW * 64];
+            const int* pw = s_done + (lane & 7) * 64 + (lane & 7);
+            int a = lds_peek(pw), b = lds_peek(pw + NW * 64);
 #define PBS_MIN_SHR(SH)                                                                  \
     {                                                                                    \
         const int a2 = __builtin_amdgcn_update_dpp(a, a, 0x110 + SH, 0xf, 0xf, false);   \
@@ -328,7 +336,7 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
                 __builtin_amdgcn_s_sleep(1);
             }
             // Cannot happen unless the protocol is broken: say so; the compute waves mark their results.
-            if (!free_now) *(volatile int*)s_fail = 1;
+            if (!free_now) lds_poke(s_fail, 1);
             wait_dma(63 - C::MAX_STEP_DMA - 1);   // the counter of outstanding loads has 6 bits
             asm volatile("" ::: "memory");
             PBS_T(8 + 4 * t + 1);
@@ -415,7 +423,7 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
         asm volatile("" : "+v"(l));
         const int er = l & 31, eh = l >> 5;
         const int m0 = (p + j * g.wg_per_group) * C::BM;
-        const bool failed = __builtin_amdgcn_readfirstlane(*(const volatile int*)s_fail) != 0;
+        const bool failed = __builtin_amdgcn_readfirstlane(lds_peek(s_fail)) != 0;
         constexpr int CW = NBW < 4 ? NBW : 4;          // block columns staged at a time
         constexpr int CHUNKS = CW * 4;                 // 16-byte pieces per staged row
         constexpr int ROWS_PER_READ = 64 / CHUNKS;     // staged rows one wave-wide read covers
@@ -456,7 +464,7 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
     // Steps whose operands have arrived from every copy wave.  The words hold the count modulo 256 and
     // are never more than the ring depth away from u, so the signed 8-bit difference is exact.
     auto producers_landed = [&](int u) -> int {
-        const int v = *(const volatile int*)(s_landed + (lane & 3) * 64 + (lane & 3));   // copy c of wave c: 4 banks
+        const int v = lds_peek(s_landed + (lane & 3) * 64 + (lane & 3));   // copy c of wave c: 4 banks
         int m = 127;
 #pragma unroll
         for (int c = 0; c < NP; ++c) {
@@ -524,9 +532,9 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
             // serves a wave's requests in order, so the reads above precede this write.
             asm volatile("" ::: "memory");
             {
-                volatile int* pd = s_done + wave * 64 + lane;   // same per-lane offset as the record reads
-                pd[0] = u + 1;
-                pd[NW * 64] = base + __popc(mask);
+                int* pd = s_done + wave * 64 + lane;   // same per-lane offset as the record reads
+                lds_poke(pd, u + 1);
+                lds_poke(pd + NW * 64, base + __popc(mask));
             }
             PBS_T(8 + 4 * u + 3);
             if (s == 0) {
