@@ -261,11 +261,6 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
                 a_voff[q] = (unsigned)r * (unsigned)a_row_bytes + a_chunk[q];
             }
             a_tile = uniform_ptr(A + (size_t)m0 * a_row_bytes);
-#ifdef PBS_EXP_SAMEA
-            a_tile = A;
-#pragma unroll
-            for (int q = 0; q < C::A_PER_WAVE; ++q) a_voff[q] = (unsigned)a_row[q] * (unsigned)a_row_bytes + a_chunk[q];
-#endif
         };
         // Issue the DMA of global step t (panel buffer `stage`, records in vrec, e0 entries before it).
         // The blocks of a step are dealt to the copy waves by entry number (dw, dw + 4, ...).
@@ -281,10 +276,7 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
             for (int k = 0; k < 2 * D16_NB / NP; ++k) {
                 const int i = dw + k * NP;
                 if (i < cnt) {
-                    unsigned id = (unsigned)__builtin_amdgcn_readlane(vrec, i);
-#ifdef PBS_EXP_SAMEW
-                    id &= 63u;
-#endif
+                    const unsigned id = (unsigned)__builtin_amdgcn_readlane(vrec, i);
                     const unsigned char* bsrc = uniform_ptr(D + ((size_t)id << 11));
                     const unsigned bdst = lds_b + (((unsigned)(e0 + i) & (RB - 1)) << 11);
                     dma16(bdst, bsrc, b_voff[0]);
