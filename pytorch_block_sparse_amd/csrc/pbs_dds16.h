@@ -332,7 +332,11 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
             wait_dma(63 - C::MAX_STEP_DMA - 1);   // the counter of outstanding loads has 6 bits
             asm volatile("" ::: "memory");
             PBS_T(8 + 4 * t + 1);
+#ifdef PBS_EXP_NODMA
+            const int n_t = 0;
+#else
             const int n_t = issue_step(stage, vrec, e0, cnt);
+#endif
             stage += C::PANEL_BYTES;
             if (stage == stage_end) stage -= RS * C::PANEL_BYTES;
             if (++sn == ns) {
@@ -489,37 +493,42 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
             if (++s == ns) s = 0;
             vrec = fetch_rec(s);   // the next step's record, needed after this step's products
             PBS_T(8 + 4 * u + 2);
+#ifndef PBS_EXP_NOCOMP
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk) {
                 const unsigned mk = (mask >> (16 * kk)) & 0xffffu;
                 const unsigned mine = (mk >> (NBW * quarter)) & ((1u << NBW) - 1u);
                 if (mine == 0) continue;
                 const int e0 = base + (kk ? __popc(mask & 0xffffu) : 0) + __popc(mk & ((1u << (NBW * quarter)) - 1u));
-                // One register index at a time keeps only 12 fragment registers live next to the 128
-                // accumulator registers.  The accumulator index stays static; the branches are wave-uniform.
-#pragma unroll
-                for (int q = 0; q < 2; ++q) {
-                    uint4 fa[TM];
-                    load_a(fa, panel, kk, q);
-                    // The blocks of this wave's columns are consecutive entries, whichever columns they
-                    // are: the next one is fetched before the products of the current one are issued
-                    // (after the last one this reads a slot whose contents are not used).
+                // The panel fragments of the k-block (both register indices) stay in registers while its
+                // blocks pass by; a block's two fragments are fetched together and feed four products, so
+                // one LDS round trip is paid per 128 matrix-core cycles (the other wave of the SIMD fills
+                // them).  The accumulator index stays static; the branches are wave-uniform.
+                {
+                    uint4 fa[2][TM];
+                    load_a(fa[0], panel, kk, 0);
+                    load_a(fa[1], panel, kk, 1);
                     int e = e0;
-                    uint4 fb_next = load_b(b_ring + (e & (RB - 1)) * C::BLK_BYTES, q);
 #pragma unroll
                     for (int jc = 0; jc < NBW; ++jc) {
                         if ((mine >> jc) & 1u) {
-                            const uint4 fb = fb_next;
+                            const unsigned char* pb = b_ring + (e & (RB - 1)) * C::BLK_BYTES;
+                            const uint4 fb0 = load_b(pb, 0);
+                            const uint4 fb1 = load_b(pb, 1);
                             ++e;
-                            fb_next = load_b(b_ring + (e & (RB - 1)) * C::BLK_BYTES, q);
 #pragma unroll
                             for (int t = 0; t < TM; ++t)
                                 acc[t][jc] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                                    __builtin_bit_cast(bf16x8, fa[t]), __builtin_bit_cast(bf16x8, fb), acc[t][jc], 0, 0, 0);
+                                    __builtin_bit_cast(bf16x8, fa[0][t]), __builtin_bit_cast(bf16x8, fb0), acc[t][jc], 0, 0, 0);
+#pragma unroll
+                            for (int t = 0; t < TM; ++t)
+                                acc[t][jc] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                                    __builtin_bit_cast(bf16x8, fa[1][t]), __builtin_bit_cast(bf16x8, fb1), acc[t][jc], 0, 0, 0);
                         }
                     }
                 }
             }
+#endif
             // this wave has read everything it needs of step u: publish (steps, entries) done.  LDS
             // serves a wave's requests in order, so the reads above precede this write.
             asm volatile("" ::: "memory");
