@@ -332,11 +332,7 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
             wait_dma(63 - C::MAX_STEP_DMA - 1);   // the counter of outstanding loads has 6 bits
             asm volatile("" ::: "memory");
             PBS_T(8 + 4 * t + 1);
-#ifdef PBS_EXP_NODMA
-            const int n_t = 0;
-#else
             const int n_t = issue_step(stage, vrec, e0, cnt);
-#endif
             stage += C::PANEL_BYTES;
             if (stage == stage_end) stage -= RS * C::PANEL_BYTES;
             if (++sn == ns) {
@@ -493,7 +489,6 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
             if (++s == ns) s = 0;
             vrec = fetch_rec(s);   // the next step's record, needed after this step's products
             PBS_T(8 + 4 * u + 2);
-#ifndef PBS_EXP_NOCOMP
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk) {
                 const unsigned mk = (mask >> (16 * kk)) & 0xffffu;
@@ -528,7 +523,6 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
                     }
                 }
             }
-#endif
             // this wave has read everything it needs of step u: publish (steps, entries) done.  LDS
             // serves a wave's requests in order, so the reads above precede this write.
             asm volatile("" ::: "memory");
