@@ -30,12 +30,15 @@ struct SddArgs {
 // mean) the rows are ranked by count and dealt to the bands in serpentine order, so that all
 // rectangles hold about the same number of blocks.  Every workgroup derives its own band from the
 // row pointer array (a few microseconds at most; above SDD_BALANCE_MAX_ROWS rows the natural order
-// is kept).  Called by all threads of the workgroup; `scratch` is LDS for nblk_r + 2 ints.
+// is kept).  Called by all threads of the workgroup; `scratch` is LDS for nblk_r + 2 ints.  Returns
+// whether the row pointers were scanned; then s_ptr_copy (if given, nblk_r + 1 ints of LDS) holds them.
 constexpr int SDD_BALANCE_MAX_ROWS = 1024;
-static __device__ __forceinline__ void sdd_band_rows(const int32_t* __restrict__ ptr, int nblk_r, int tiles_r, int band,
-                                                     int SR, int* s_rowid, int* scratch, int tid, int nthreads) {
+static __device__ __forceinline__ bool sdd_band_rows(const int32_t* __restrict__ ptr, int nblk_r, int tiles_r, int band,
+                                                     int SR, int* s_rowid, int* scratch, int tid, int nthreads,
+                                                     int* s_ptr_copy = nullptr) {
     bool skewed = false;
-    if (nblk_r <= SDD_BALANCE_MAX_ROWS && tiles_r >= 2) {
+    const bool scanned = nblk_r <= SDD_BALANCE_MAX_ROWS && tiles_r >= 2;
+    if (scanned) {
         int* s_max = scratch + nblk_r;
         int* s_sum = s_max + 1;
         if (tid == 0) {
@@ -44,7 +47,12 @@ static __device__ __forceinline__ void sdd_band_rows(const int32_t* __restrict__
         }
         __syncthreads();
         for (int r = tid; r < nblk_r; r += nthreads) {
-            const int n = ptr[r + 1] - ptr[r];
+            const int lo = ptr[r], hi = ptr[r + 1];
+            const int n = hi - lo;
+            if (s_ptr_copy) {   // saves the caller a second trip to global memory
+                s_ptr_copy[r] = lo;
+                if (r == nblk_r - 1) s_ptr_copy[nblk_r] = hi;
+            }
             scratch[r] = n;
             atomicMax(s_max, n);
             atomicAdd(s_sum, n);
@@ -72,6 +80,7 @@ static __device__ __forceinline__ void sdd_band_rows(const int32_t* __restrict__
         }
         __syncthreads();
     }
+    return scanned;
 }
 
 template <typename T, int SR, int SC, int QW, int NW>

@@ -83,7 +83,6 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
     const int band = tile / a.tiles_c, grp = tile % a.tiles_c;
     const int nblk_c = a.K / 32;
     const int nunits = (nblk_c + 1) / 2;
-    sdd_band_rows(a.ptr, nblk_r, a.tiles_r, band, SR, s_rowid, reinterpret_cast<int*>(smem), tid, C::NT);
     // scratch in the (not yet used) chunk buffers
     constexpr int EMAX = 8192, UMAX = 1024;
     int* s_lo = reinterpret_cast<int*>(smem);   // [SR] first entry of each row
@@ -92,11 +91,24 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
     int* s_eblk = s_ecol + EMAX;                // [EMAX] data block of each cached entry
     int* s_cnt = s_eblk + EMAX;                 // [UMAX] blocks of the band per column unit
     int* s_ug = s_cnt + UMAX;                   // [UMAX] rectangle * 8 + place of each column unit
-    static_assert((2 * SR + 1 + 2 * EMAX + 2 * UMAX) * 4 <= NS * C::STAGE_BYTES, "scratch fits in the chunk buffers");
+    int* s_scan = s_ug + UMAX;                  // [SDD_BALANCE_MAX_ROWS + 2] scratch of the row scan
+    int* s_ptr_copy = s_scan + SDD_BALANCE_MAX_ROWS + 2;   // [SDD_BALANCE_MAX_ROWS + 1] row pointers, if scanned
+    static_assert((2 * SR + 1 + 2 * EMAX + 2 * UMAX + 2 * SDD_BALANCE_MAX_ROWS + 3) * 4 <= NS * C::STAGE_BYTES,
+                  "scratch fits in the chunk buffers");
+    const bool have_ptr = sdd_band_rows(a.ptr, nblk_r, a.tiles_r, band, SR, s_rowid, s_scan, tid, C::NT, s_ptr_copy);
     __syncthreads();
     if (tid < SR) {
         const int r = s_rowid[tid];
-        const int lo = r >= 0 ? a.ptr[r] : 0, hi = r >= 0 ? a.ptr[r + 1] : 0;
+        int lo = 0, hi = 0;
+        if (r >= 0) {
+            if (have_ptr) {
+                lo = s_ptr_copy[r];
+                hi = s_ptr_copy[r + 1];
+            } else {
+                lo = a.ptr[r];
+                hi = a.ptr[r + 1];
+            }
+        }
         s_lo[tid] = lo;
         s_rs[tid + 1] = hi - lo;
     }
@@ -116,13 +128,15 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
     const bool dealt = cached && nunits <= UMAX && a.tiles_c >= 2;
     int my_lo = 0, my_n = 0;
     if (cached) {
-        for (int r = 0; r < SR; ++r) {
-            const int lo = s_lo[r], off = s_rs[r], n = s_rs[r + 1] - off;
-            for (int i = tid; i < n; i += C::NT) {
-                const int2 e = *reinterpret_cast<const int2*>(a.idx + 2 * (size_t)(lo + i));
-                s_ecol[off + i] = e.x;
-                s_eblk[off + i] = e.y;
-            }
+        // one sweep over the band's entries (entry i belongs to the row r with s_rs[r] <= i < s_rs[r + 1]):
+        // all loads of a thread are in flight together
+        for (int i = tid; i < nent; i += C::NT) {
+            int r = 0;
+#pragma unroll
+            for (int k = 1; k < SR; ++k) r += (i >= s_rs[k]) ? 1 : 0;
+            const int2 e = *reinterpret_cast<const int2*>(a.idx + 2 * (size_t)(s_lo[r] + i - s_rs[r]));
+            s_ecol[i] = e.x;
+            s_eblk[i] = e.y;
         }
         if (dealt)
             for (int u = tid; u < nunits; u += C::NT) s_cnt[u] = 0;
