@@ -40,37 +40,22 @@ struct SddBf16Cfg {
     static_assert(NS_ >= 2 && NS_ <= 4, "chunk buffers");
 };
 
-template <int QW, int TC_, int NS_>
-__global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
-    using C = SddBf16Cfg<QW, TC_, NS_>;
-    constexpr int NS = C::NS;
-    constexpr int SR = C::SR, SC = C::SC, NW = C::NW, TC = C::TC;
-
-    extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-    int* s_blk = reinterpret_cast<int*>(smem + NS * C::STAGE_BYTES);                  // [LIST_MAX] data block
-    unsigned short* s_pos = reinterpret_cast<unsigned short*>(s_blk + C::LIST_MAX);  // [LIST_MAX] (rl << 8) | cl
-    int* s_rowoff = reinterpret_cast<int*>(s_pos + C::LIST_MAX);                     // [SR + 1]
-    const unsigned lds0 = (unsigned)(uintptr_t)smem;
-
-    const int ntiles = a.tiles_r * a.tiles_c;
-    const int wg = xcd_tile_id(blockIdx.x, ntiles * a.nsplit);
-    if (wg < 0) return;
-    const int sp = wg / ntiles;
-    const int tile = wg % ntiles;
-    const int c0 = (tile % a.tiles_c) * SC;
-    const int nblk_r = a.N / 32;
-
+// The rectangle's rows, columns and block list, built by all threads of the workgroup (NT threads, of
+// which the first 8 waves place the blocks).  smem: scratch of at least SDD_BF16_PROLOGUE_BYTES at the start
+// of the (not yet used) chunk buffers.  Results in LDS: s_blk / s_pos (data block and (row place << 8 |
+// column place) of each block, row-major), s_rowoff[SR] = number of blocks, s_rowid[SR] = block row of
+// W in each row place or -1, s_gu[SC / 2] = column unit (pair of block columns) in each place or -1.
+constexpr int SDD_BF16_EMAX = 8192, SDD_BF16_UMAX = 1024;
+constexpr int SDD_BF16_PROLOGUE_BYTES = (2 * 16 + 1 + 2 * SDD_BF16_EMAX + 2 * SDD_BF16_UMAX + 2 * SDD_BALANCE_MAX_ROWS + 3) * 4;
+template <int NT>
+static __device__ __forceinline__ void sdd_bf16_prologue(const SddArgs& a, int tile, unsigned char* smem, int* s_blk,
+                                                         unsigned short* s_pos, int* s_rowoff, int* s_rowid, int* s_gu) {
+    constexpr int SR = 16, SC = 16, NW = 8;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int lrow = lane & 31;
-    const int h = lane >> 5;
-
-#ifdef PBS_EXP_TIMING
-    const bool prof_on = (wg == 100) && (lane == 0) && (wave == 0);
-    const int prof_base = 0;
-#endif
-    PBS_T(0);
+    const int c0 = (tile % a.tiles_c) * SC;
+    const int nblk_r = a.N / 32;
     // ---- which rows and columns of W this rectangle covers, and the list of its blocks (row-major) ----
     // Rows: the band's 16 block rows (sdd_band_rows).  Columns: normally the band's columns c0 .. c0+15.
     // When the band's entries fit in LDS the columns of the band are instead dealt to the band's
@@ -78,13 +63,11 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
     // the units are ranked by their number of blocks in this band and handed out in serpentine order.
     // Rectangles of one band then hold the same number of blocks to within a few, instead of
     // 64 +- 7 at density 0.25, and the kernel no longer waits for its fullest rectangle.
-    int* s_rowid = s_rowoff + SR + 2;   // [SR] block row of W in each place of this rectangle's band, or -1
-    int* s_gu = s_rowid + SR;           // [SC / 2] column unit in each place of this rectangle, or -1
     const int band = tile / a.tiles_c, grp = tile % a.tiles_c;
     const int nblk_c = a.K / 32;
     const int nunits = (nblk_c + 1) / 2;
     // scratch in the (not yet used) chunk buffers
-    constexpr int EMAX = 8192, UMAX = 1024;
+    constexpr int EMAX = SDD_BF16_EMAX, UMAX = SDD_BF16_UMAX;
     int* s_lo = reinterpret_cast<int*>(smem);   // [SR] first entry of each row
     int* s_rs = s_lo + SR;                      // [SR + 1] start of each row's entries in the cached arrays
     int* s_ecol = s_rs + SR + 1;                // [EMAX] block column of each cached entry
@@ -93,9 +76,7 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
     int* s_ug = s_cnt + UMAX;                   // [UMAX] rectangle * 8 + place of each column unit
     int* s_scan = s_ug + UMAX;                  // [SDD_BALANCE_MAX_ROWS + 2] scratch of the row scan
     int* s_ptr_copy = s_scan + SDD_BALANCE_MAX_ROWS + 2;   // [SDD_BALANCE_MAX_ROWS + 1] row pointers, if scanned
-    static_assert((2 * SR + 1 + 2 * EMAX + 2 * UMAX + 2 * SDD_BALANCE_MAX_ROWS + 3) * 4 <= NS * C::STAGE_BYTES,
-                  "scratch fits in the chunk buffers");
-    const bool have_ptr = sdd_band_rows(a.ptr, nblk_r, a.tiles_r, band, SR, s_rowid, s_scan, tid, C::NT, s_ptr_copy);
+    const bool have_ptr = sdd_band_rows(a.ptr, nblk_r, a.tiles_r, band, SR, s_rowid, s_scan, tid, NT, s_ptr_copy);
     __syncthreads();
     if (tid < SR) {
         const int r = s_rowid[tid];
@@ -130,7 +111,7 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
     if (cached) {
         // one sweep over the band's entries (entry i belongs to the row r with s_rs[r] <= i < s_rs[r + 1]):
         // all loads of a thread are in flight together
-        for (int i = tid; i < nent; i += C::NT) {
+        for (int i = tid; i < nent; i += NT) {
             int r = 0;
 #pragma unroll
             for (int k = 1; k < SR; ++k) r += (i >= s_rs[k]) ? 1 : 0;
@@ -139,15 +120,15 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
             s_eblk[i] = e.y;
         }
         if (dealt)
-            for (int u = tid; u < nunits; u += C::NT) s_cnt[u] = 0;
+            for (int u = tid; u < nunits; u += NT) s_cnt[u] = 0;
         __syncthreads();
         if (dealt) {
-            for (int i = tid; i < nent; i += C::NT) {
+            for (int i = tid; i < nent; i += NT) {
                 const int c = s_ecol[i];
                 if (c >= 0 && c < nblk_c) atomicAdd(&s_cnt[c >> 1], 1);
             }
             __syncthreads();
-            for (int u = tid; u < nunits; u += C::NT) {
+            for (int u = tid; u < nunits; u += NT) {
                 const int n = s_cnt[u];
                 int rank = 0;
                 for (int o = 0; o < nunits; ++o) {
@@ -173,6 +154,7 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
         };
 #pragma unroll
         for (int rr = 0; rr < SR / NW; ++rr) {
+            if (wave >= NW) break;
             const int r = wave * (SR / NW) + rr;
             const int off = s_rs[r], n = s_rs[r + 1] - off;
             int cnt = 0;
@@ -222,6 +204,7 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
         };
 #pragma unroll
         for (int rr = 0; rr < SR / NW; ++rr) {
+            if (wave >= NW) break;
             const int r = wave * (SR / NW) + rr;
             const int off = s_rs[r], n = s_rs[r + 1] - off;
             int run = s_rowoff[r];
@@ -249,6 +232,42 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
         }
     }
     __syncthreads();
+}
+
+template <int QW, int TC_, int NS_>
+__global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
+    using C = SddBf16Cfg<QW, TC_, NS_>;
+    constexpr int NS = C::NS;
+    constexpr int SR = C::SR, SC = C::SC, NW = C::NW, TC = C::TC;
+
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+    int* s_blk = reinterpret_cast<int*>(smem + NS * C::STAGE_BYTES);                  // [LIST_MAX] data block
+    unsigned short* s_pos = reinterpret_cast<unsigned short*>(s_blk + C::LIST_MAX);  // [LIST_MAX] (rl << 8) | cl
+    int* s_rowoff = reinterpret_cast<int*>(s_pos + C::LIST_MAX);                     // [SR + 1]
+    const unsigned lds0 = (unsigned)(uintptr_t)smem;
+
+    const int ntiles = a.tiles_r * a.tiles_c;
+    const int wg = xcd_tile_id(blockIdx.x, ntiles * a.nsplit);
+    if (wg < 0) return;
+    const int sp = wg / ntiles;
+    const int tile = wg % ntiles;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lrow = lane & 31;
+    const int h = lane >> 5;
+
+#ifdef PBS_EXP_TIMING
+    const bool prof_on = (wg == 100) && (lane == 0) && (wave == 0);
+    const int prof_base = 0;
+#endif
+    PBS_T(0);
+    // ---- which rows and columns of W this rectangle covers, and the list of its blocks (row-major) ----
+    int* s_rowid = s_rowoff + SR + 2;   // [SR] block row of W in each place of this rectangle's band, or -1
+    int* s_gu = s_rowid + SR;           // [SC / 2] column unit in each place of this rectangle, or -1
+    static_assert(SDD_BF16_PROLOGUE_BYTES <= NS * C::STAGE_BYTES, "scratch fits in the chunk buffers");
+    const int nblk_c = a.K / 32;
+    sdd_bf16_prologue<C::NT>(a, tile, smem, s_blk, s_pos, s_rowoff, s_rowid, s_gu);
     const int nq = __builtin_amdgcn_readfirstlane(s_rowoff[SR]);
     if (nq == 0) return;
     PBS_T(1);
