@@ -180,6 +180,9 @@ __global__ __launch_bounds__(256) void dds_plan_kernel(const int32_t* __restrict
     }
 }
 
+// Development aid, not part of the product build: with -DPBS_EXP_TIMING one or two waves of one workgroup
+// stamp the cycle counter at the phase boundaries of their loops (PBS_T), and pbs_debug_read_prof copies
+// the stamps out.  Without the macro PBS_T compiles to nothing.
 #ifdef PBS_EXP_TIMING
 __device__ long long g_prof[8192];
 #define PBS_T(slot) do { if (prof_on) g_prof[prof_base + (slot)] = (long long)__builtin_readcyclecounter(); } while (0)
