@@ -53,16 +53,11 @@ struct Elem<bf16_t> {
                                                           __builtin_bit_cast(bf16x8, b[q]), acc, 0, 0, 0);
         }
     }
-    // round to nearest even, NaN kept quiet
+    // round to nearest even, NaN kept quiet: the hardware conversion (v_cvt_pk_bf16_f32, two values per
+    // instruction where the compiler can pair them)
     static __device__ __forceinline__ bf16_t from_f32(float v) {
-        uint32_t u = __float_as_uint(v);
         bf16_t r;
-        if ((u & 0x7fffffffu) > 0x7f800000u) {
-            r.bits = (uint16_t)((u >> 16) | 0x40u);
-        } else {
-            u += 0x7fffu + ((u >> 16) & 1u);
-            r.bits = (uint16_t)(u >> 16);
-        }
+        r.bits = __builtin_bit_cast(uint16_t, static_cast<__bf16>(v));
         return r;
     }
     static __device__ __forceinline__ float to_f32(bf16_t v) { return __uint_as_float(((uint32_t)v.bits) << 16); }
