@@ -425,11 +425,20 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
 #pragma unroll
         for (int cg = 0; cg < NBW / CW; ++cg) {   // CW block columns at a time
             float bv[CW];
+            {
+                bf16_t braw[CW];   // all loads first: one wait
 #pragma unroll
-            for (int jc = 0; jc < CW; ++jc) {
-                const int col = col0 + (cg * CW + jc) * 32 + er;
-                bv[jc] = (bias && col < g.N) ? E::to_f32(bias[col]) : 0.f;
-                if (gave_up || failed) bv[jc] = __builtin_nanf("");
+                for (int jc = 0; jc < CW; ++jc) {
+                    const int col = col0 + (cg * CW + jc) * 32 + er;
+                    braw[jc].bits = 0;
+                    if (bias) braw[jc] = bias[col < g.N ? col : 0];
+                }
+#pragma unroll
+                for (int jc = 0; jc < CW; ++jc) {
+                    const int col = col0 + (cg * CW + jc) * 32 + er;
+                    bv[jc] = col < g.N ? E::to_f32(braw[jc]) : 0.f;
+                    if (gave_up || failed) bv[jc] = __builtin_nanf("");
+                }
             }
             const int col = col0 + cg * CW * 32 + rd_c;
 #pragma unroll
@@ -441,11 +450,15 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
 #pragma unroll
                         for (int vv = 0; vv < 4; ++vv)
                             st_w[vv * C::STAGE_ROW + jc * 32] = E::from_f32(acc[t][cg * CW + jc][4 * gq + vv] + bv[jc]);
+                    // both reads first: one wait for the staged rows instead of one per store
+                    uint4 val[8 / ROWS_PER_READ];
+#pragma unroll
+                    for (int pp = 0; pp < 8 / ROWS_PER_READ; ++pp)
+                        val[pp] = *reinterpret_cast<const uint4*>(st_r + pp * ROWS_PER_READ * C::STAGE_ROW);
 #pragma unroll
                     for (int pp = 0; pp < 8 / ROWS_PER_READ; ++pp) {
-                        const uint4 val = *reinterpret_cast<const uint4*>(st_r + pp * ROWS_PER_READ * C::STAGE_ROW);
                         const int row = m0 + (ms * TM + t) * 32 + gq * 8 + pp * ROWS_PER_READ + rd_r;
-                        if (row < g.M && col < g.N) *reinterpret_cast<uint4*>(out + (size_t)row * g.N + col) = val;
+                        if (row < g.M && col < g.N) *reinterpret_cast<uint4*>(out + (size_t)row * g.N + col) = val[pp];
                     }
                 }
             }
