@@ -87,6 +87,7 @@ class BlockSparseMatrixBase(torch.nn.Module):
         self.register_buffer("col_start_ends_b", col_start_ends_b)
         self.register_buffer("blocks", blocks)
         self._plans = {}
+        self.validate_indices()
         self.check_ = False
         if callback:
             self.updated_data()
@@ -295,6 +296,73 @@ class BlockSparseMatrixBase(torch.nn.Module):
             theirs = dense_version[r * bs0 : (r + 1) * bs0, c * bs1 : (c + 1) * bs1]
             if not (mine == theirs).all():
                 raise Exception("non matching data")
+
+    def validate_indices(self):
+        """Check the five index buffers against each other and against ``data``; raise on the first mismatch.
+
+        Runs where index buffers enter the object: at the end of ``rebuild`` (where the reference calls
+        ``sanity_check`` on both compressed lists, block_sparse.py:67-73) and after ``load_state_dict``.
+        It covers ``sanity_check``'s conditions (:431-463) and, beyond them, that the start/end lists start
+        at 0 and never decrease and that the data-block ids of each list are a permutation of
+        ``0..nnz-1``: the kernels index ``data`` and the entry lists with these values.  Shapes and dtypes
+        are checked on the host; the value checks run on the buffers' device and are read back once.
+        """
+        bs0, bs1 = self.block_shape
+        X, Y = self.blocks_count()
+        nnz = self.data.shape[0] // bs0
+        it = self.int_type
+        lists = (
+            ("cols_a", self.cols_a, "row_start_ends_a", self.row_start_ends_a, X, Y),
+            ("rows_b", self.rows_b, "col_start_ends_b", self.col_start_ends_b, Y, X),
+        )
+        for name, ids, ends_name, ends, n_lists, _ in lists:
+            if ids.dim() != 2 or tuple(ids.shape) != (nnz, 2):
+                raise Exception("%s should have shape (%d, 2), not %s" % (name, nnz, tuple(ids.shape)))
+            if ids.dtype != it:
+                raise Exception("%s should be %s, not of type %s" % (name, it, ids.dtype))
+            if ends.dim() != 1 or ends.shape[0] != n_lists + 1:
+                raise Exception("%s should have shape (%d,), not %s" % (ends_name, n_lists + 1, tuple(ends.shape)))
+            if ends.dtype != it:
+                raise Exception("%s should be %s, not of type %s" % (ends_name, it, ends.dtype))
+        blocks = self.blocks
+        if blocks.dim() != 1 or blocks.shape[0] != 2 * nnz or blocks.dtype != it:
+            raise Exception("blocks should be %s of shape (%d,), not %s %s" % (it, 2 * nnz, blocks.dtype, tuple(blocks.shape)))
+        problems = []   # (message, 0-d bool tensor: True = broken)
+        for name, ids, ends_name, ends, _, limit in lists:
+            e = ends.long()
+            problems.append(("%s should start at 0 and never decrease" % ends_name, (e[0] != 0) | (e[1:] < e[:-1]).any()))
+            problems.append(("%s last element should be equal to the block count (%d)" % (ends_name, nnz), e[-1] != nnz))
+            if nnz:
+                c, b = ids[:, 0].long(), ids[:, 1].long()
+                problems.append(("%s holds a block coordinate outside [0, %d)" % (name, limit), (c.min() < 0) | (c.max() >= limit)))
+                b_ok = (b >= 0) & (b < nnz)
+                seen = torch.zeros(nnz, dtype=torch.long, device=ids.device)
+                seen.index_add_(0, b.clamp(0, nnz - 1), b_ok.long())
+                problems.append(
+                    ("the data block ids of %s should be a permutation of 0..%d" % (name, nnz - 1), (seen != 1).any())
+                )
+        if nnz:
+            b2 = blocks.view(-1, 2).long()
+            problems.append((
+                "blocks holds a block position outside the %d x %d grid" % (X, Y),
+                (b2.min() < 0) | (b2[:, 0].max() >= Y) | (b2[:, 1].max() >= X),
+            ))
+        flags = torch.stack([p[1].to(self.blocks.device) for p in problems]).tolist()
+        for (message, _), broken in zip(problems, flags):
+            if broken:
+                raise Exception(message)
+
+    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+        """Index buffers copied in from a checkpoint are validated before any kernel reads them."""
+        super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
+        error_msgs = args[4] if len(args) > 4 else kwargs.get("error_msgs")
+        self._plans = {}
+        try:
+            self.validate_indices()
+        except Exception as e:  # reported the way torch reports the other problems of a state dict
+            if error_msgs is None:
+                raise
+            error_msgs.append("%sindex buffers are inconsistent: %s" % (prefix, e))
 
     def sanity_check(self, cols, row_end, shape, block_shape):
         """Consistency of one compressed list.  reference: block_sparse.py:431-463."""

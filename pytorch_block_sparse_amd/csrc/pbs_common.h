@@ -67,6 +67,10 @@ struct Elem<bf16_t> {
 // the column is (lane & 31).
 static __device__ __forceinline__ int acc_row(int v, int h) { return 8 * (v >> 2) + 4 * h + (v & 3); }
 
+// A row/column pointer value read from a caller's index array, forced into [0, nnz]: a corrupt
+// pointer array then selects wrong entries instead of reading outside the entry list.
+static __device__ __forceinline__ int clamp_entry(int v, int nnz) { return v < 0 ? 0 : (v > nnz ? nnz : v); }
+
 static __device__ __forceinline__ uint4 ldg16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
 
 // Two 16-byte rows of 8 bf16 (row k even, row k odd, same 8 columns) -> 8 words, word n holding
@@ -111,7 +115,7 @@ static __device__ __forceinline__ void dma16(unsigned lds_base_uniform, const un
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t"
                  :
                  : "s"(lds_base_uniform), "v"(voff), "s"(base_uniform)
-                 : "memory");
+                 : "memory", "m0");
 }
 
 // wait until at most n (wave-uniform) of this wave's DMA loads are outstanding, make this wave's
@@ -135,7 +139,7 @@ static __device__ __forceinline__ void dma4(unsigned lds_base_uniform, const uns
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2\n\t"
                  :
                  : "s"(lds_base_uniform), "v"(voff), "s"(base_uniform)
-                 : "memory");
+                 : "memory", "m0");
 }
 
 // wait until at most n (wave-uniform) of this wave's DMA loads are outstanding

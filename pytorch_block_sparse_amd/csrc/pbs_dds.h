@@ -121,8 +121,8 @@ __global__ __launch_bounds__(256) void dds_plan_kernel(const int32_t* __restrict
         const int c = slots[blockIdx.x * NB + tid];
         const bool ok = c >= 0 && c < nblk_n;
         s_col[tid] = ok ? c : -1;
-        s_lo[tid] = ok ? ptr[c] : 0;
-        s_hi[tid] = ok ? ptr[c + 1] : 0;
+        s_lo[tid] = ok ? clamp_entry(ptr[c], nnz) : 0;
+        s_hi[tid] = ok ? clamp_entry(ptr[c + 1], nnz) : 0;
     }
     __syncthreads();
     int nk = 0, ne = 0;   // running totals (kept by every thread of wave 0)
@@ -180,15 +180,6 @@ __global__ __launch_bounds__(256) void dds_plan_kernel(const int32_t* __restrict
     }
 }
 
-// Development aid, not part of the product build: with -DPBS_EXP_TIMING one or two waves of one workgroup
-// stamp the cycle counter at the phase boundaries of their loops (PBS_T), and pbs_debug_read_prof copies
-// the stamps out.  Without the macro PBS_T compiles to nothing.
-#ifdef PBS_EXP_TIMING
-__device__ long long g_prof[8192];
-#define PBS_T(slot) do { if (prof_on) g_prof[prof_base + (slot)] = (long long)__builtin_readcyclecounter(); } while (0)
-#else
-#define PBS_T(slot) do { } while (0)
-#endif
 
 struct DdsArgs {
     const void* a;         // [M, K] row-major
@@ -329,10 +320,6 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
         return end - cum_s <= RB;
     };
 
-#ifdef PBS_EXP_TIMING
-    const bool prof_on = (tile == 300) && (lane == 0) && (wave == 0 || wave == NW);
-    const int prof_base = wave == 0 ? 0 : 4096;
-#endif
     const unsigned char* A_tile = static_cast<const unsigned char*>(g.a) + (size_t)m0 * g.K * E::ESZ;
     const unsigned char* D = static_cast<const unsigned char*>(g.data);
 
@@ -430,13 +417,11 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
                 next = s + 1;
                 vrec = fetch_recs(next);
             }
-            PBS_T(8 + 4 * s + 0);
             const int vends = fetch_ends(s);
             int later = 0;   // DMA of the steps after s may stay in flight
 #pragma unroll
             for (int k = 1; k < RS; ++k) later += pend[k];
             wait_dma_and_barrier(later);
-            PBS_T(8 + 4 * s + 1);
             unpack_ends(ce, vends);
 #pragma unroll
             for (int k = 0; k + 1 < RS; ++k) pend[k] = pend[k + 1];
@@ -449,9 +434,7 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
                     ++next;
                     vrec = fetch_recs(next);
                 }
-            PBS_T(8 + 4 * s + 2);
             compute(s);
-            PBS_T(8 + 4 * s + 3);
             cum_s = ce.c0;
         }
         drain_barrier();   // the rings are reused by the epilogue
@@ -565,7 +548,6 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
         }
     };
 
-    PBS_T(0);
     if constexpr (NP == 0) {
         copy_loop(wave, [&](int s) {
             load_step_recs(s);
@@ -582,22 +564,16 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
                 lds_barrier();
                 next = s + 1;
             }
-            PBS_T(8 + 4 * s + 0);
             const int vends = fetch_ends(s);
             load_step_recs(s);
             lds_barrier();
             unpack_ends(ce, vends);
-            PBS_T(8 + 4 * s + 1);
             if (s > 0)
                 while (can_issue(next, s, cum_s, ce)) ++next;
-            PBS_T(8 + 4 * s + 2);
             compute_step(s);
-            PBS_T(8 + 4 * s + 3);
             cum_s = ce.c0;
         }
-        PBS_T(1);
         lds_barrier();
-        PBS_T(2);
     }
 
     // ---- epilogue: each wave passes its 32 x 128 sub-tiles through its own LDS region so that the
@@ -639,7 +615,6 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
-    PBS_T(3);
 }
 
 }  // namespace pbs

@@ -63,7 +63,7 @@ __global__ __launch_bounds__(256) void dds16_plan_kernel(const int32_t* __restri
     int* rec = out + R;
     if (tid <= NB) {
         const int nb = nb0 + tid;
-        s_ptr[tid] = ptr[nb < nblk_n ? nb : nblk_n];
+        s_ptr[tid] = clamp_entry(ptr[nb < nblk_n ? nb : nblk_n], nnz);
     }
     __syncthreads();
     const int e_begin = s_ptr[0], e_end = s_ptr[NB];
@@ -209,11 +209,6 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
     const int ns = __builtin_amdgcn_readfirstlane(s_plan[0]);   // steps (k-pairs) per tile
     const int ne = __builtin_amdgcn_readfirstlane(s_plan[1]);   // entries per tile
     const int nsteps = ns * ntiles;                              // global steps of this workgroup
-#ifdef PBS_EXP_TIMING
-    const bool prof_on = (wg == 100) && (lane == 0) && (wave == 0 || wave == NW);
-    const int prof_base = wave == 0 ? 0 : 4096;
-#endif
-    PBS_T(0);
 
     // lane l: int l of the record of step s of a tile
     auto fetch_rec = [&](int s) -> int { return s_plan[(1 + s) * R + lane]; };
@@ -312,7 +307,6 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
         const unsigned stage_end = stage + RS * C::PANEL_BYTES;
         enter_tile(0);
         for (int t = 0; t < nsteps; ++t) {
-            PBS_T(8 + 4 * t + 0);
             // wait until the panel buffer and the block slots of step t are free
             const int cnt = __popc((unsigned)__builtin_amdgcn_readlane(vrec, D16_F_MASK));
             const int e0 = jn * ne + __builtin_amdgcn_readlane(vrec, D16_F_CUM);
@@ -331,7 +325,6 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
             if (!free_now) lds_poke(s_fail, 1);
             wait_dma(63 - C::MAX_STEP_DMA - 1);   // the counter of outstanding loads has 6 bits
             asm volatile("" ::: "memory");
-            PBS_T(8 + 4 * t + 1);
             const int n_t = issue_step(stage, vrec, e0, cnt);
             stage += C::PANEL_BYTES;
             if (stage == stage_end) stage -= RS * C::PANEL_BYTES;
@@ -341,11 +334,9 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
                 if (t + 1 < nsteps) enter_tile(jn);
             }
             vrec = fetch_rec(sn);   // consumed in the next iteration: the LDS latency is hidden
-            PBS_T(8 + 4 * t + 2);
             // behind the operands of step t: the number t + 1 (mod 256) onto this wave's landed words
             dma4(landed_lds, uniform_ptr(reinterpret_cast<const unsigned char*>(g.seq + ((t + 1) & 255))), 0u);
             (void)n_t;
-            PBS_T(8 + 4 * t + 3);
         }
         wait_dma(0);
         return;
@@ -483,7 +474,6 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
         int landed = 0;
         int vrec = fetch_rec(0);
         for (int u = 0; u < nsteps; ++u) {
-            PBS_T(8 + 4 * u + 0);
             if (landed <= u) {
                 for (int spin = 0; spin < C::SPIN_LIMIT; ++spin) {
                     landed = producers_landed(u);
@@ -495,13 +485,11 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
                 if (landed <= u) gave_up = true;
             }
             asm volatile("" ::: "memory");   // operand reads stay behind the poll
-            PBS_T(8 + 4 * u + 1);
             const unsigned mask = (unsigned)__builtin_amdgcn_readlane(vrec, D16_F_MASK);
             const int base = j * ne + __builtin_amdgcn_readlane(vrec, D16_F_CUM);
             const unsigned char* panel = a_ring + (u % RS) * C::PANEL_BYTES;
             if (++s == ns) s = 0;
             vrec = fetch_rec(s);   // the next step's record, needed after this step's products
-            PBS_T(8 + 4 * u + 2);
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk) {
                 const unsigned mk = (mask >> (16 * kk)) & 0xffffu;
@@ -544,7 +532,6 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
                 lds_poke(pd, u + 1);
                 lds_poke(pd + NW * 64, base + __popc(mask));
             }
-            PBS_T(8 + 4 * u + 3);
             if (s == 0) {
                 epilogue(j);
                 zero_acc();

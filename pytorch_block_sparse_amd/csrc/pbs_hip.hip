@@ -223,12 +223,6 @@ extern "C" {
 
 int pbs_abi_version(void) { return PBS_ABI_VERSION; }
 
-#ifdef PBS_EXP_TIMING
-int pbs_debug_read_prof(long long* host, int n) {
-    hipDeviceSynchronize();
-    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_prof), (size_t)n * 8);
-}
-#endif
 
 const char* pbs_error_string(int code) {
     switch (code) {

@@ -33,7 +33,7 @@ struct SddArgs {
 // is kept).  Called by all threads of the workgroup; `scratch` is LDS for nblk_r + 2 ints.  Returns
 // whether the row pointers were scanned; then s_ptr_copy (if given, nblk_r + 1 ints of LDS) holds them.
 constexpr int SDD_BALANCE_MAX_ROWS = 1024;
-static __device__ __forceinline__ bool sdd_band_rows(const int32_t* __restrict__ ptr, int nblk_r, int tiles_r, int band,
+static __device__ __forceinline__ bool sdd_band_rows(const int32_t* __restrict__ ptr, int nnz, int nblk_r, int tiles_r, int band,
                                                      int SR, int* s_rowid, int* scratch, int tid, int nthreads,
                                                      int* s_ptr_copy = nullptr) {
     bool skewed = false;
@@ -47,8 +47,8 @@ static __device__ __forceinline__ bool sdd_band_rows(const int32_t* __restrict__
         }
         __syncthreads();
         for (int r = tid; r < nblk_r; r += nthreads) {
-            const int lo = ptr[r], hi = ptr[r + 1];
-            const int n = hi - lo;
+            const int lo = clamp_entry(ptr[r], nnz), hi = clamp_entry(ptr[r + 1], nnz);
+            const int n = hi > lo ? hi - lo : 0;
             if (s_ptr_copy) {   // saves the caller a second trip to global memory
                 s_ptr_copy[r] = lo;
                 if (r == nblk_r - 1) s_ptr_copy[nblk_r] = hi;
@@ -141,11 +141,11 @@ __global__ __launch_bounds__(NW * 64) void sdd_kernel(SddArgs a) {
     // ---- list the nonzero blocks of the rectangle, row-major ----
     int my_lo = 0, my_n = 0;
     __shared__ int s_rowid[SR];   // block row of W in each place of this rectangle's band, or -1
-    sdd_band_rows(a.ptr, nblk_r, a.tiles_r, tr, SR, s_rowid, reinterpret_cast<int*>(smem), tid, NT);
+    sdd_band_rows(a.ptr, a.nnz, nblk_r, a.tiles_r, tr, SR, s_rowid, reinterpret_cast<int*>(smem), tid, NT);
     if (tid < SR) {
         const int r = s_rowid[tid];
         if (r >= 0) {
-            int lo = a.ptr[r], hi = a.ptr[r + 1];
+            const int lo = clamp_entry(a.ptr[r], a.nnz), hi = clamp_entry(a.ptr[r + 1], a.nnz);
             // rows are sorted by block column: first entry with column >= c0
             int l = lo, u = hi;
             while (l < u) {

@@ -76,7 +76,7 @@ static __device__ __forceinline__ void sdd_bf16_prologue(const SddArgs& a, int t
     int* s_ug = s_cnt + UMAX;                   // [UMAX] rectangle * 8 + place of each column unit
     int* s_scan = s_ug + UMAX;                  // [SDD_BALANCE_MAX_ROWS + 2] scratch of the row scan
     int* s_ptr_copy = s_scan + SDD_BALANCE_MAX_ROWS + 2;   // [SDD_BALANCE_MAX_ROWS + 1] row pointers, if scanned
-    const bool have_ptr = sdd_band_rows(a.ptr, nblk_r, a.tiles_r, band, SR, s_rowid, s_scan, tid, NT, s_ptr_copy);
+    const bool have_ptr = sdd_band_rows(a.ptr, a.nnz, nblk_r, a.tiles_r, band, SR, s_rowid, s_scan, tid, NT, s_ptr_copy);
     __syncthreads();
     if (tid < SR) {
         const int r = s_rowid[tid];
@@ -86,12 +86,12 @@ static __device__ __forceinline__ void sdd_bf16_prologue(const SddArgs& a, int t
                 lo = s_ptr_copy[r];
                 hi = s_ptr_copy[r + 1];
             } else {
-                lo = a.ptr[r];
-                hi = a.ptr[r + 1];
+                lo = clamp_entry(a.ptr[r], a.nnz);
+                hi = clamp_entry(a.ptr[r + 1], a.nnz);
             }
         }
         s_lo[tid] = lo;
-        s_rs[tid + 1] = hi - lo;
+        s_rs[tid + 1] = hi > lo ? hi - lo : 0;
     }
     if (tid < SC / 2) s_gu[tid] = -1;
     __syncthreads();
@@ -172,7 +172,7 @@ static __device__ __forceinline__ void sdd_bf16_prologue(const SddArgs& a, int t
         if (tid < SR) {
             const int r = s_rowid[tid];
             if (r >= 0) {
-                const int lo = a.ptr[r], hi = a.ptr[r + 1];
+                const int lo = clamp_entry(a.ptr[r], a.nnz), hi = clamp_entry(a.ptr[r + 1], a.nnz);
                 int l = lo, u = hi;
                 while (l < u) {   // rows are sorted by block column: first entry with column >= c0
                     const int mid = (l + u) >> 1;
@@ -257,11 +257,6 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
     const int lrow = lane & 31;
     const int h = lane >> 5;
 
-#ifdef PBS_EXP_TIMING
-    const bool prof_on = (wg == 100) && (lane == 0) && (wave == 0);
-    const int prof_base = 0;
-#endif
-    PBS_T(0);
     // ---- which rows and columns of W this rectangle covers, and the list of its blocks (row-major) ----
     int* s_rowid = s_rowoff + SR + 2;   // [SR] block row of W in each place of this rectangle's band, or -1
     int* s_gu = s_rowid + SR;           // [SC / 2] column unit in each place of this rectangle, or -1
@@ -270,7 +265,6 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
     sdd_bf16_prologue<C::NT>(a, tile, smem, s_blk, s_pos, s_rowoff, s_rowid, s_gu);
     const int nq = __builtin_amdgcn_readfirstlane(s_rowoff[SR]);
     if (nq == 0) return;
-    PBS_T(1);
 
     const int t_begin = sp * a.tokens_per_split;
     int t_end = t_begin + a.tokens_per_split;
@@ -398,24 +392,19 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
             for (int k = 0; k < NS - 1; ++k)
                 if (k < nchunks) pend[k] = issue_chunk(k);
             for (int ci = 0; ci < nchunks; ++ci) {
-                PBS_T(8 + 4 * ci + 0);
                 int later = 0;
 #pragma unroll
                 for (int k = 1; k < NS; ++k) later += pend[k];
                 // chunk ci has landed for every wave, and every wave is done reading chunk ci - 1
                 wait_dma_and_barrier(later);
-                PBS_T(8 + 4 * ci + 1);
 #pragma unroll
                 for (int k = 0; k + 1 < NS; ++k) pend[k] = pend[k + 1];
                 pend[NS - 1] = 0;
                 if (ci + NS - 1 < nchunks) pend[NS - 2] = issue_chunk(ci + NS - 1);   // into the buffer of chunk ci - 1
-                PBS_T(8 + 4 * ci + 2);
                 compute_chunk(ci);
-                PBS_T(8 + 4 * ci + 3);
             }
             lds_barrier();   // the next pass refills the buffers
         }
-        PBS_T(2);
 
         // ---- store: result row j (X feature), column i (G feature) ----
 #pragma unroll
@@ -429,7 +418,6 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
                 }
             }
         }
-        PBS_T(3);
     }
 }
 

@@ -14,8 +14,7 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# PBS_HIP_LIBRARY selects another build of the same library (kernel experiments)
-LIB_PATH = os.environ.get("PBS_HIP_LIBRARY") or os.path.join(_HERE, "csrc", "libpbs_hip.so")
+LIB_PATH = os.path.join(_HERE, "csrc", "libpbs_hip.so")
 
 DTYPE_CODES = {torch.float32: 0, torch.bfloat16: 1}
 SUPPORTED_DTYPES = tuple(DTYPE_CODES)

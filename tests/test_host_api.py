@@ -177,6 +177,49 @@ def test_state_dict_round_trip():
         assert torch.equal(getattr(a.weight, k), getattr(b.weight, k))
 
 
+def test_corrupt_index_buffers_are_rejected():
+    """Index buffers are validated where they enter (the reference runs sanity_check on both compressed
+    lists in every rebuild, block_sparse.py:67-73, :431-463): a checkpoint whose lists are inconsistent
+    raises from load_state_dict instead of reaching a kernel."""
+    np.random.seed(0)
+    torch.manual_seed(0)
+    a = BlockSparseLinear(64, 128, True, density=0.5, device="cpu")
+    good = {k: v.clone() for k, v in a.state_dict().items()}
+    nnz = a.weight.cols_a.shape[0]
+
+    def corrupt(key, fn):
+        sd = {k: v.clone() for k, v in good.items()}
+        fn(sd["weight." + key])
+        return sd
+
+    cases = {
+        "row list runs past the entries": corrupt("row_start_ends_a", lambda t: t.__setitem__(-1, nnz + 5)),
+        "row list decreases": corrupt("row_start_ends_a", lambda t: t.__setitem__(1, nnz + 1)),
+        "column list does not start at 0": corrupt("col_start_ends_b", lambda t: t.__setitem__(0, 1)),
+        "block column out of range": corrupt("cols_a", lambda t: t.__setitem__((0, 0), 99)),
+        "negative block row": corrupt("rows_b", lambda t: t.__setitem__((0, 0), -1)),
+        "data block id out of range": corrupt("cols_a", lambda t: t.__setitem__((0, 1), nnz)),
+        "data block id used twice": corrupt("rows_b", lambda t: t.__setitem__((0, 1), int(t[1, 1]))),
+        "block position outside the grid": corrupt("blocks", lambda t: t.__setitem__(0, 1000)),
+    }
+    for what, sd in cases.items():
+        b = BlockSparseLinear(64, 128, True, density=0.5, device="cpu")
+        with pytest.raises(RuntimeError, match="index buffers are inconsistent"):
+            b.load_state_dict(sd)
+        # direct use of the check on the module that now holds the bad buffers
+        with pytest.raises(Exception):
+            b.weight.validate_indices()
+    b = BlockSparseLinear(64, 128, True, density=0.5, device="cpu")
+    b.load_state_dict(good)   # the untouched state dict still loads
+    b.weight.validate_indices()
+    # sanity_check keeps the reference's signature and conditions
+    w = b.weight
+    w.sanity_check(w.cols_a, w.row_start_ends_a, w.shape, w.block_shape)
+    w.sanity_check(w.rows_b, w.col_start_ends_b, (w.shape[1], w.shape[0]), (32, 32))
+    with pytest.raises(Exception, match="row_end last element"):
+        w.sanity_check(w.cols_a[:-1], w.row_start_ends_a, w.shape, w.block_shape)
+
+
 class _Tiny(torch.nn.Module):
     def __init__(self):
         super().__init__()
