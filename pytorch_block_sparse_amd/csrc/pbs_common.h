@@ -110,12 +110,15 @@ static __device__ __forceinline__ const unsigned char* uniform_ptr(const unsigne
     return reinterpret_cast<const unsigned char*>(((uint64_t)hi << 32) | lo);
 }
 
-// one DMA instruction: lane p copies the 16 bytes at base + voff to LDS chunk (lds_base/16 + p)
+// one DMA instruction: lane p copies the 16 bytes at base + voff to LDS chunk (lds_base/16 + p).
+// M0 is written inside the statement and cannot be named as a clobber (the compiler treats it as a
+// reserved register and rejects that with a warning about undefined behaviour); these kernels contain
+// nothing else that makes the compiler use M0 (no LDS-DMA builtins, no dynamically indexed registers).
 static __device__ __forceinline__ void dma16(unsigned lds_base_uniform, const unsigned char* base_uniform, unsigned voff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t"
                  :
                  : "s"(lds_base_uniform), "v"(voff), "s"(base_uniform)
-                 : "memory", "m0");
+                 : "memory");
 }
 
 // wait until at most n (wave-uniform) of this wave's DMA loads are outstanding, make this wave's
@@ -139,7 +142,7 @@ static __device__ __forceinline__ void dma4(unsigned lds_base_uniform, const uns
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2\n\t"
                  :
                  : "s"(lds_base_uniform), "v"(voff), "s"(base_uniform)
-                 : "memory", "m0");
+                 : "memory");
 }
 
 // wait until at most n (wave-uniform) of this wave's DMA loads are outstanding
