@@ -115,6 +115,10 @@ int pbs_blocksparse_matmul(const void* dense_a, const void* data, const void* pl
  *   both row-major contiguous.  The pattern is given by the CSR pair
  *   (row_start_ends_a, cols_a) instead of the reference's `blocks` list so that a
  *   workgroup can find the blocks of its tile of W without scanning all of them.
+ *   A caller of the reference's entry point has the pair at hand: the object that owns
+ *   `blocks` registers row_start_ends_a and cols_a as buffers next to it
+ *   (block_sparse.py:58-65), built from the same mask by build_indices (:125-153); a
+ *   caller that holds nothing but a mask obtains all of them from pbs_build_indices.
  *   Every token is accumulated (the reference drops tokens % 32 when tokens > 32).
  *   `out` need not be zeroed.
  *

@@ -105,3 +105,21 @@ def test_build_indices_argument_checks(lib):
     assert f(p, null, 4, 4, 17, p, p, p, p, p, p, null) == ERR_SHAPE
     assert f(null, null, 4, 4, 2, p, p, p, p, p, p, null) == ERR_NULL
     assert f(p, null, 4, 4, 2, null, p, p, p, p, p, null) == ERR_NULL
+
+
+def test_reference_side_binding_matches_the_header(lib):
+    """include/pbs_hip_ctypes.py is the binding a maintainer of the reference would use: its prototypes must be
+    those the package's own binding declares, and its error path must raise on a rejected call."""
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location("pbs_hip_ctypes", os.path.join(ROOT, "include", "pbs_hip_ctypes.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    for name, (restype, argtypes) in mod.PROTOTYPES.items():
+        assert name in native._PROTOTYPES, name
+        r2, a2 = native._PROTOTYPES[name]
+        assert restype is r2 and list(argtypes) == list(a2), name
+    b = mod.PbsHip(native.LIB_PATH)
+    assert b.lib.pbs_abi_version() == lib.pbs_abi_version()
+    with pytest.raises(RuntimeError, match="pbs:"):
+        b._check(b.lib.pbs_blocksparse_matmul(None, None, None, None, None, 4, 64, 64, 1, 1, 0, None), "matmul")
