@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define PBS_ABI_VERSION 2
+#define PBS_ABI_VERSION 3
 #define PBS_BLOCK 32
 
 /* element type of dense operands, packed data and results (accumulation is fp32) */
@@ -44,6 +44,7 @@ extern "C" {
 #define PBS_ERR_MISALIGNED (-4)    /* a dense/data pointer is not 16-byte aligned */
 #define PBS_ERR_WORKSPACE (-5)     /* workspace/plan buffer missing, misaligned or too small */
 #define PBS_ERR_TOO_LARGE (-6)     /* a size exceeds what the kernels index with */
+#define PBS_ERR_SCRATCH (-7)       /* more scratch needed than the built-in buffer of the no-allocation entry point */
 
 int pbs_abi_version(void);
 const char* pbs_error_string(int code);
@@ -134,6 +135,31 @@ int pbs_blocksparse_matmul_back(const void* dense_a, const void* dense_b,
                                 void* data_out,
                                 int64_t tokens, int out_features, int in_features, int nnz,
                                 int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * pbs_blocksparse_matmul_back for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  Same arguments, same kernels and bit-identical results as pbs_blocksparse_matmul_back,
+ * without the workspace pair: the fp32 partial sums of a split token range go to a device array of
+ * PBS_NOALLOC_SCRATCH_BYTES (64 MiB) that is part of the library (every GPU the library is used on
+ * holds its own copy until the process ends).  The call makes no hipMalloc/hipFree and calls no
+ * allocating routine.
+ *
+ *   - A problem whose pbs_blocksparse_matmul_back_workspace_bytes() exceeds the array is rejected
+ *     with PBS_ERR_SCRATCH before anything is launched (4096 x 4096 at density 0.25 with 16384
+ *     tokens in bf16 needs exactly 64 MiB and fits).
+ *   - Nothing in the array has to be cleared between calls: every word the reduction kernel reads
+ *     is written by the product kernel of the same call first.
+ *   - All calls on one GPU share that GPU's array, whatever their stream: two calls that overlap on
+ *     one GPU race.  Order them on one stream, or use the workspace entry point for concurrent work.
+ */
+#define PBS_NOALLOC_SCRATCH_BYTES (64u << 20)
+size_t pbs_blocksparse_matmul_back_noalloc_max_bytes(void);
+int pbs_blocksparse_matmul_back_noalloc(const void* dense_a, const void* dense_b,
+                                        const int32_t* row_start_ends_a, const int32_t* cols_a,
+                                        void* data_out,
+                                        int64_t tokens, int out_features, int in_features, int nnz,
+                                        int dtype, void* stream);
 
 #ifdef __cplusplus
 }

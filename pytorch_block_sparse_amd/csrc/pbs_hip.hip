@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <mutex>
 
 #include "pbs_common.h"
 #include "pbs_dds.h"
@@ -215,6 +216,34 @@ static int launch_sdd(SddArgs a, int dtype, void* workspace, size_t workspace_by
     return rc;
 }
 
+// ---- scratch of the entry point that allocates nothing ----
+// One device array per GPU, part of the library's code object: it exists on every GPU the library runs on
+// from the moment the code object is loaded there until the process ends.  Host code never uses the
+// array's name as an address (on the host it only stands for the symbol): the address on a device is
+// asked for once, with that device current, and kept.
+static __device__ __align__(256) unsigned char scratch[PBS_NOALLOC_SCRATCH_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+static void* g_scratch_ptr[MAX_DEVICES];
+static std::mutex g_scratch_mutex;
+
+static int scratch_of_current_device(void** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= MAX_DEVICES) return PBS_ERR_TOO_LARGE;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return PBS_ERR_WORKSPACE;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return PBS_OK;
+}
+
 }  // namespace pbs
 
 using namespace pbs;
@@ -233,6 +262,7 @@ const char* pbs_error_string(int code) {
         case PBS_ERR_MISALIGNED: return "pbs: dense/data pointers must be 16-byte aligned";
         case PBS_ERR_WORKSPACE: return "pbs: workspace missing, misaligned or too small";
         case PBS_ERR_TOO_LARGE: return "pbs: size exceeds the kernels' index range";
+        case PBS_ERR_SCRATCH: return "pbs: the problem needs more scratch than the library's built-in buffer holds; use the entry point that takes a workspace";
         default: break;
     }
     if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
@@ -352,6 +382,22 @@ int pbs_blocksparse_matmul_back(const void* dense_a, const void* dense_b, const 
     a.tiles_r = a.tiles_c = a.nsplit = a.tokens_per_split = 0;
     if (dtype == PBS_DTYPE_F32) return launch_sdd<float>(a, dtype, workspace, workspace_bytes, s);
     return launch_sdd<bf16_t>(a, dtype, workspace, workspace_bytes, s);
+}
+
+size_t pbs_blocksparse_matmul_back_noalloc_max_bytes(void) { return PBS_NOALLOC_SCRATCH_BYTES; }
+
+int pbs_blocksparse_matmul_back_noalloc(const void* dense_a, const void* dense_b, const int32_t* row_start_ends_a,
+                                        const int32_t* cols_a, void* data_out, int64_t tokens, int out_features,
+                                        int in_features, int nnz, int dtype, void* stream) {
+    // what pbs_blocksparse_matmul_back would ask the caller for (0 for arguments it is going to reject itself)
+    const size_t need = pbs_blocksparse_matmul_back_workspace_bytes(tokens, out_features, in_features, nnz, dtype);
+    if (need > (size_t)PBS_NOALLOC_SCRATCH_BYTES) return PBS_ERR_SCRATCH;
+    void* ws = nullptr;
+    if (need > 0) {
+        if (int rc = scratch_of_current_device(&ws)) return rc;
+    }
+    return pbs_blocksparse_matmul_back(dense_a, dense_b, row_start_ends_a, cols_a, data_out, tokens, out_features,
+                                       in_features, nnz, dtype, ws, need, stream);
 }
 
 }  // extern "C"

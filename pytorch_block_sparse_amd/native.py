@@ -37,6 +37,8 @@ _PROTOTYPES = {
         _i32,
         [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _vp, ctypes.c_size_t, _vp],
     ),
+    "pbs_blocksparse_matmul_back_noalloc_max_bytes": (ctypes.c_size_t, []),
+    "pbs_blocksparse_matmul_back_noalloc": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _vp]),
 }
 
 EXPORTED_SYMBOLS = tuple(_PROTOTYPES)
