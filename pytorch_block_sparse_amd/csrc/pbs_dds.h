@@ -193,19 +193,25 @@ struct DdsArgs {
 
 // TRANS = 0: B[k][n] = block[k*32 + n]   (forward: the packed block is W_block^T = [in][out])
 // TRANS = 1: B[k][n] = block[n*32 + k]   (dX: contraction runs along the packed block's rows)
-template <typename T, int TRANS, int TM, int SK, int RS, int RB, int NP, int NBW_ = DDS_NBW>
+template <typename T, int TRANS, int TM, int SK, int RS, int RB, int NP, int NBW_ = DDS_NBW, int NSL_ = 4>
 struct DdsCfg {
     using E = Elem<T>;
     static constexpr int NW = DDS_NW;                    // compute waves
-    // Block columns per compute wave: 4 (the tile covers its whole group of 8 block columns) or 2 (the
-    // tile covers half a group; twice as many, half as wide tiles for results with few columns).
+    // The 8 compute waves are NSL token slices x NH = 8 / NSL column parts of NBW block columns each:
+    //   NSL = 4, NBW = 4   the tile covers its whole group of 8 block columns (two halves);
+    //   NSL = 4, NBW = 2   the tile covers half a group: twice as many, half as wide tiles;
+    //   NSL = 8, NBW = 8   every wave has all 8 block columns and its own 32 * TM tokens: all waves do
+    //                      the same products, so the barrier per step costs nothing however uneven the
+    //                      pattern is (with column halves a step lasts as long as its fuller half).
     static constexpr int NBW = NBW_;
-    static constexpr int NSUB = DDS_NBW / NBW_;          // tiles per column group
-    static constexpr int TILE_COLS = 2 * NBW_;           // block columns per tile
-    static_assert(NBW_ == 4 || NBW_ == 2, "block columns per wave");
+    static constexpr int NSL = NSL_;
+    static constexpr int NH = DDS_NW / NSL_;
+    static constexpr int TILE_COLS = NH * NBW_;          // block columns per tile
+    static constexpr int NSUB = DDS_NB / TILE_COLS;      // tiles per column group
+    static_assert((NSL_ == 4 && (NBW_ == 4 || NBW_ == 2)) || (NSL_ == 8 && NBW_ == 8), "wave layout");
     static constexpr int ND = NP ? NP : NW;              // waves that issue DMA
     static constexpr int NT = (NW + NP) * 64;
-    static constexpr int BM = 4 * TM * 32;
+    static constexpr int BM = NSL_ * TM * 32;
     static constexpr int ROWB = 32 * E::ESZ;             // bytes of one 32-wide operand row
     static constexpr int CPR = ROWB / 16;                // 16-byte chunks per row (4 or 8)
     static constexpr int RPI = 64 / CPR;                 // rows filled by one DMA instruction (16 or 8)
@@ -219,8 +225,10 @@ struct DdsCfg {
     static constexpr int A_RING_BYTES = RS * STEP_BYTES;
     static constexpr int B_RING_BYTES = RB * BLK_BYTES;
     static constexpr int RING_BYTES = A_RING_BYTES + B_RING_BYTES;
-    // the epilogue stages one 32-row x 128-column sub-tile per compute wave through LDS
-    static constexpr int EPI_WAVE_BYTES = 32 * NBW_ * 32 * E::ESZ;
+    // the epilogue stages 8 result rows of a compute wave's columns at a time through LDS (rows padded by
+    // 16 bytes: the two lane halves write rows 4 apart, which would otherwise meet in the same banks)
+    static constexpr int EPI_ROW_BYTES = NBW_ * 32 * E::ESZ + 16;
+    static constexpr int EPI_WAVE_BYTES = 8 * EPI_ROW_BYTES;
     static constexpr int EPI_BYTES = NW * EPI_WAVE_BYTES;
     static constexpr int WORK_BYTES = RING_BYTES > EPI_BYTES ? RING_BYTES : EPI_BYTES;   // + the plan records
     static_assert(PANEL_INSTR % ND == 0 && A_PER_WAVE >= 1, "panel DMA must divide evenly over the issuing waves");
@@ -236,9 +244,9 @@ static __device__ __forceinline__ int swz(int r) {
     return CPR == 4 ? ((r >> 2) & 3) : ((r >> 1) & 7);
 }
 
-template <typename T, int TRANS, int TM, int SK, int RS, int RB, int NP, int NBW_ = DDS_NBW>
+template <typename T, int TRANS, int TM, int SK, int RS, int RB, int NP, int NBW_ = DDS_NBW, int NSL_ = 4>
 __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
-    using C = DdsCfg<T, TRANS, TM, SK, RS, RB, NP, NBW_>;
+    using C = DdsCfg<T, TRANS, TM, SK, RS, RB, NP, NBW_, NSL_>;
     using E = typename C::E;
     constexpr int NBW = C::NBW, NW = DDS_NW, ND = C::ND, NQ = E::NQ, CPR = C::CPR, R = DDS_REC_INTS;
 
@@ -450,8 +458,8 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
     // =====================================================================================
     // compute side
     // =====================================================================================
-    const int ms = wave & 3;            // token slice
-    const int half = (wave >> 2) & 1;   // block-column half of the tile
+    const int ms = wave % C::NSL;       // token slice
+    const int half = wave / C::NSL;     // block-column part of the tile
     const int col_w = col_lo + half * NBW;   // first of this wave's columns within the group
     const int lrow = lane & 31;
     const int h = lane >> 5;
@@ -576,8 +584,8 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
         lds_barrier();
     }
 
-    // ---- epilogue: each wave passes its 32 x 128 sub-tiles through its own LDS region so that the
-    //      global stores are 16 bytes per lane along rows; bias fused ----
+    // ---- epilogue: each wave passes its results, 8 rows at a time, through its own LDS region (inside the
+    //      rings, which are idle now) so that the global stores are 16 bytes per lane along rows; bias fused ----
     T* out = static_cast<T*>(g.out);
     const T* bias = static_cast<const T*>(g.bias);
     unsigned char* epi = smem + wave * C::EPI_WAVE_BYTES;
@@ -593,27 +601,34 @@ __global__ __launch_bounds__((DDS_NW + NP) * 64) void dds_kernel(DdsArgs g) {
     constexpr int WCOLS = NBW * 32;                        // result columns of one wave
     constexpr int CHUNKS_PER_ROW = WCOLS / EPL;            // 16-byte chunks per staged row
     constexpr int ROWS_PER_PASS = 64 / CHUNKS_PER_ROW;     // rows stored by one wave instruction
+    constexpr int PASSES = 8 / ROWS_PER_PASS;              // store instructions per 8 staged rows
+    static_assert(ROWS_PER_PASS >= 1 && 8 % ROWS_PER_PASS == 0, "8 staged rows are stored in whole passes");
+    const int rd_r = lane / CHUNKS_PER_ROW, rd_c = (lane % CHUNKS_PER_ROW) * EPL;
+    int cid = colid[0];   // the block column this lane's chunk belongs to
+#pragma unroll
+    for (int j = 1; j < NBW; ++j) cid = (rd_c >= j * 32) ? colid[j] : cid;
+    const int col = cid * 32 + (rd_c & 31);
 #pragma unroll
     for (int t = 0; t < TM; ++t) {
-        T* e_t = reinterpret_cast<T*>(epi);
-#pragma unroll
-        for (int j = 0; j < NBW; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) e_t[acc_row(v, h) * WCOLS + j * 32 + lrow] = E::from_f32(acc[t][j][v] + bv[j]);
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         const int rbase = m0 + (ms * TM + t) * 32;
 #pragma unroll
-        for (int p = 0; p < 32 / ROWS_PER_PASS; ++p) {
-            const int r = p * ROWS_PER_PASS + lane / CHUNKS_PER_ROW;
-            const int c = (lane % CHUNKS_PER_ROW) * EPL;
-            const uint4 val = *reinterpret_cast<const uint4*>(epi + (r * WCOLS + c) * E::ESZ);
-            int cid = colid[0];   // the block column this lane's chunk belongs to
+        for (int gq = 0; gq < 4; ++gq) {   // rows 8 gq .. 8 gq + 7 of the 32
 #pragma unroll
-            for (int j = 1; j < NBW; ++j) cid = (c >= j * 32) ? colid[j] : cid;
-            const int row = rbase + r, col = cid * 32 + (c & 31);
-            if (row < g.M && cid >= 0) *reinterpret_cast<uint4*>(out + (size_t)row * g.N + col) = val;
+            for (int j = 0; j < NBW; ++j)
+#pragma unroll
+                for (int vv = 0; vv < 4; ++vv)
+                    *reinterpret_cast<T*>(epi + (4 * h + vv) * C::EPI_ROW_BYTES + (j * 32 + lrow) * E::ESZ) =
+                        E::from_f32(acc[t][j][4 * gq + vv] + bv[j]);
+            uint4 val[PASSES];   // all reads first: one wait for the staged rows
+#pragma unroll
+            for (int p = 0; p < PASSES; ++p)
+                val[p] = *reinterpret_cast<const uint4*>(epi + (p * ROWS_PER_PASS + rd_r) * C::EPI_ROW_BYTES + rd_c * E::ESZ);
+#pragma unroll
+            for (int p = 0; p < PASSES; ++p) {
+                const int row = rbase + gq * 8 + p * ROWS_PER_PASS + rd_r;
+                if (row < g.M && cid >= 0) *reinterpret_cast<uint4*>(out + (size_t)row * g.N + col) = val[p];
+            }
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
 }
 

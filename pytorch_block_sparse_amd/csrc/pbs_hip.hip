@@ -37,11 +37,11 @@ static int raise_lds_limit(K kernel, int bytes, std::atomic<uint64_t>& done) {
     return 0;
 }
 
-template <typename T, int TRANS, int TM, int SK, int RS, int RB, int NP, int NBW = DDS_NBW>
+template <typename T, int TRANS, int TM, int SK, int RS, int RB, int NP, int NBW = DDS_NBW, int NSL = 4>
 static int launch_dds(DdsArgs g, hipStream_t stream) {
-    using C = DdsCfg<T, TRANS, TM, SK, RS, RB, NP, NBW>;
+    using C = DdsCfg<T, TRANS, TM, SK, RS, RB, NP, NBW, NSL>;
     static std::atomic<uint64_t> done{0};
-    auto kernel = dds_kernel<T, TRANS, TM, SK, RS, RB, NP, NBW>;
+    auto kernel = dds_kernel<T, TRANS, TM, SK, RS, RB, NP, NBW, NSL>;
     constexpr int LDS_MAX = 160 * 1024;
     // rings (or the epilogue staging) plus this group's plan records
     const size_t lds = (size_t)C::WORK_BYTES + (size_t)g.group_ints * sizeof(int);
@@ -53,6 +53,10 @@ static int launch_dds(DdsArgs g, hipStream_t stream) {
     hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)tiles)), dim3(C::NT), lds, stream, g);
     return (int)hipGetLastError();
 }
+
+#ifndef PBS_SHAPE3_FACTOR
+#define PBS_SHAPE3_FACTOR 0.8
+#endif
 
 // ---- wide-tile persistent bf16 kernel ----
 // The plan buffer holds the narrow plan first, then (when k is a multiple of 64) the wide one.
@@ -115,23 +119,54 @@ static int launch_dds16(const DdsArgs& g, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
-// Tile shapes: 256 tokens x 8 block columns when that still gives every CU a tile, else 128 tokens x 8,
-// else (results with few columns) 128 tokens x 4 block columns.
+// Tile shapes: 256 tokens x 8 block columns, 128 x 8, or 128 x 4 (twice as many, half as wide tiles).
+// One workgroup runs per CU, so a launch takes ceil(tiles / 256) rounds of one tile time each; the shape
+// with the smallest rounds x tile area wins (smaller tiles move more operand bytes per product, hence the
+// small handicaps), e.g. 384 tiles of 128 x 8 take two rounds, of which the second is half empty, while
+// the same problem in 768 tiles of 128 x 4 takes three full rounds of half the length.  A shape whose
+// rings and plan records do not fit in LDS (very long contractions) is skipped.
 // bf16 steps cover two k-blocks (the matrix cores go through a k-block 16x faster than in fp32).
 template <typename T, int TRANS>
 static int dispatch_dds(const DdsArgs& g, hipStream_t stream) {
-    const long long big_tiles = (long long)((g.M + 255) / 256) * g.n_groups;
-    const long long mid_tiles = (long long)((g.M + 127) / 128) * g.n_groups;
-    if constexpr (sizeof(T) == 4) {
-        if (big_tiles >= 256) return launch_dds<T, TRANS, 2, 1, 3, 8, 0>(g, stream);
-        if (mid_tiles >= 160) return launch_dds<T, TRANS, 1, 1, 3, 8, 0>(g, stream);
-        return launch_dds<T, TRANS, 1, 1, 3, 8, 0, 2>(g, stream);
-    } else {
+    if constexpr (sizeof(T) == 2) {
         if (wide_kernel_fits(g.M, g.N, g.K)) return launch_dds16<TRANS>(g, stream);
-        if (big_tiles >= 256) return launch_dds<T, TRANS, 2, 2, 3, 16, 4>(g, stream);
-        if (mid_tiles >= 160) return launch_dds<T, TRANS, 1, 2, 3, 16, 4>(g, stream);
-        return launch_dds<T, TRANS, 1, 2, 3, 16, 4, 2>(g, stream);
     }
+    // shapes: 0 = 256 x 8 (4 token slices x 2 column halves), 1 = 128 x 8, 2 = 128 x 4,
+    //         3 = 256 x 8 with 8 token slices (every wave has all 8 columns; fp32 only: 8 accumulators of fp32
+    //             fragments fit the registers, and balanced waves are worth more than the larger fragments cost)
+    constexpr int NSHAPES = sizeof(T) == 4 ? 4 : 3;
+    const long long tiles[4] = {
+        (long long)((g.M + 255) / 256) * g.n_groups,
+        (long long)((g.M + 127) / 128) * g.n_groups,
+        (long long)((g.M + 127) / 128) * g.n_groups * 2,
+        (long long)((g.M + 255) / 256) * g.n_groups,
+    };
+    const double area[4] = {2048.0, 1024.0 * 1.04, 512.0 * 1.10, 2048.0 * PBS_SHAPE3_FACTOR};
+    double cost[4];
+    for (int c = 0; c < NSHAPES; ++c) cost[c] = (double)((tiles[c] + 255) / 256) * area[c];
+    int order[4] = {0, 1, 2, 3};
+    for (int i = 0; i < NSHAPES; ++i)
+        for (int j = i + 1; j < NSHAPES; ++j)
+            if (cost[order[j]] < cost[order[i]]) {
+                const int t = order[i];
+                order[i] = order[j];
+                order[j] = t;
+            }
+    int rc = PBS_ERR_TOO_LARGE;
+    for (int i = 0; i < NSHAPES && rc == PBS_ERR_TOO_LARGE; ++i) {
+        const int c = order[i];
+        if constexpr (sizeof(T) == 4) {
+            rc = c == 0 ? launch_dds<T, TRANS, 2, 1, 3, 8, 0>(g, stream)
+                 : c == 1 ? launch_dds<T, TRANS, 1, 1, 3, 8, 0>(g, stream)
+                 : c == 2 ? launch_dds<T, TRANS, 1, 1, 3, 8, 0, 2>(g, stream)
+                          : launch_dds<T, TRANS, 1, 1, 3, 8, 0, 8, 8>(g, stream);
+        } else {
+            rc = c == 0 ? launch_dds<T, TRANS, 2, 2, 3, 16, 4>(g, stream)
+                 : c == 1 ? launch_dds<T, TRANS, 1, 2, 3, 16, 4>(g, stream)
+                          : launch_dds<T, TRANS, 1, 2, 3, 16, 4, 2>(g, stream);
+        }
+    }
+    return rc;
 }
 
 // ---- sparse-output product ----

@@ -237,3 +237,18 @@ def test_uneven_rows_use_balanced_column_groups(cuda, dtype):
     yb = m.reverse_matmul(x.to(cuda), True, bias=bias.to(cuda))
     assert_close(yb, to64(x) @ w_dense.T + to64(bias)[None, :], dtype, "uneven rows fwd + bias")
     assert torch.equal(yb[:, 12 * 32:], bias.to(cuda)[None, 12 * 32:].expand(tokens, -1))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_long_contraction(cuda, dtype):
+    """A contraction of 32768 features (a 4096 -> 32000-class layer's input gradient): the schedule records of a
+    column group no longer fit in LDS beside the larger tile shapes' rings, and the library has to fall
+    through to a shape that fits instead of refusing (the reference has no such limit)."""
+    big, small, tokens = 32768, 64, 40
+    np.random.seed(17)
+    # out = big: the input gradient contracts over 32768; in = big: the forward does
+    for out_f, in_f in ((big, small), (small, big)):
+        n_blocks = 96
+        print(f"long contraction {in_f}->{out_f} {dtype}", flush=True)
+        m = _matrix(out_f, in_f, None, n_blocks, dtype, cuda, seed=17)
+        _check_all(m, (tokens,), dtype, cuda, 17, f"{in_f}->{out_f}")
