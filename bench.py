@@ -6,9 +6,15 @@ sparse support, for BlockSparseLinear(4096 -> 4096, density 0.25), 16384 tokens,
 with fp32 accumulation.  Inputs are synthetic (seeded) and resident in HBM before timing starts.
 
 Prints ONE JSON line: effective TFLOP/s (2*M*nnz*1024 per GEMM, 3 GEMMs per step) with
-  roofline      the slowest of the three kernels against the MI355X dense bf16 MFMA peak,
-  dense         the same three GEMMs dense through torch.matmul (hipBLASLt) at the same shape,
-  cpu_baseline  the CPU dense-equivalent path (oracle) timed on the host cores on a token sample.
+  roofline       the slowest of the three kernels against the MI355X dense MFMA peak of the dtype,
+  dense_hipblaslt  the same three GEMMs dense through torch.matmul (hipBLASLt) at the same shape,
+  cpu_baseline   the CPU dense-equivalent path (oracle) timed on the host cores, full size,
+  other_configs  the other benchmark configurations (1024->256 forward, the two RoBERTa feed-forward
+                 shapes in fp32, the RoBERTa-base training step), each with its own dense comparison.
+
+Timing: after a settling phase and `--warmup` untimed steps, exactly `--steps` steps are timed between two
+synchronisations; an event is recorded after every kernel of every timed step.  `ms_per_step` and `value`
+are the median over the timed steps (the mean over the same region is `ms_per_step_mean`).
 """
 import argparse
 import json
@@ -20,21 +26,40 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}  # MI355X dense matrix peaks
+HBM_TBPS = 8.0
 
-# HBM bytes per launch (fetch + write) of each kernel, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE runs of this script, scaled by what the same counters read for a plain 256 MiB device
-# copy (fetch x2.0, write x1.0).  Counters cannot be read from inside the process, so the figures
-# are recorded here per workload and token count; other workloads report null.
-MIB = float(1 << 20)
-MEASURED_TRAFFIC = {
-    ("c4_4096x4096_d0.25_bf16", 16384): {
-        "fwd": (413.5 + 128.0) * MIB,
-        "dx": (385.5 + 128.0) * MIB,
-        "dw": (385.8 + 64.0 + 64.0 + 8.0) * MIB,   # partial sums, then the reduction
-    },
-}
+# HBM bytes per launch (fetch + write) of each kernel come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this script (counters cannot be read from inside the process).  They are kept in profiles/traffic.json
+# together with a hash of the kernel sources they were measured on; a figure measured on other sources is
+# not reported (null).
 BASELINE_WORKLOAD = "c4_4096x4096_d0.25_bf16"
-BASELINE_METRIC = "effective TFLOP/s fwd+bwd at 4096\u00b2 d=0.25; % of MFMA peak; vs dense GEMM"   # as in BASELINE.json
+BASELINE_METRIC = "effective TFLOP/s fwd+bwd at 4096² d=0.25; % of MFMA peak; vs dense GEMM"   # as in BASELINE.json
+OTHER_LAYER_WORKLOADS = ("c1_1024x256_d0.1_fp32", "c2_768x3072_d0.5_fp32", "c3_3072x768_d0.25_zipf_fp32")
+ROBERTA_WORKLOAD = "c5_roberta_base_mlm_fp32"
+
+
+def kernel_source_hash():
+    """sha256 over the kernel sources, in name order."""
+    import glob
+    import hashlib
+
+    h = hashlib.sha256()
+    src = os.path.join(ROOT, "pytorch_block_sparse_amd", "csrc")
+    for path in sorted(glob.glob(os.path.join(src, "*.h")) + glob.glob(os.path.join(src, "*.hip"))):
+        h.update(os.path.basename(path).encode())
+        h.update(open(path, "rb").read())
+    return h.hexdigest()
+
+
+def measured_traffic(workload, tokens, kernel):
+    """Bytes per launch from profiles/traffic.json, or None if absent or measured on other kernel sources."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    if not os.path.exists(path):
+        return None
+    rec = json.load(open(path))
+    if rec.get("kernel_source_sha256") != kernel_source_hash():
+        return None
+    return rec.get("bytes_per_launch", {}).get(f"{workload}@{tokens}", {}).get(kernel)
 
 
 def parse():
@@ -46,37 +71,66 @@ def parse():
     p.add_argument("--tokens", type=int, default=None, help="override the workload's token count")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     p.add_argument("--no-dense", action="store_true", help="skip the dense hipBLASLt leg")
-    p.add_argument("--cpu-sample-tokens", type=int, default=2048)
+    p.add_argument("--no-others", action="store_true", help="skip the other_configs leg (C1, C2, C3, RoBERTa step)")
+    p.add_argument("--cpu-sample-tokens", type=int, default=None, help="tokens of the CPU baseline leg (default: all)")
     p.add_argument("--copy-calibration", action="store_true",
                    help="also run a plain 256 MiB device copy (reference point for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     return p.parse_args()
 
 
-def time_gpu(fn, steps, warmup):
-    """Average milliseconds per call of fn over `steps` calls, HIP events on the current stream."""
+def median(v):
+    v = sorted(v)
+    n = len(v)
+    return v[n // 2] if n % 2 else 0.5 * (v[n // 2 - 1] + v[n // 2])
+
+
+def settle(fn, seconds=0.3):
+    """Untimed: run fn until `seconds` have passed, so that clocks and caches are past their start-up transient."""
     import torch
 
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+
+
+def time_steps(kernels, steps, warmup):
+    """kernels: ordered {name: callable}.  Returns (median ms per step, mean ms per step, median ms per kernel)."""
+    import torch
+
+    def step():
+        for f in kernels.values():
+            f()
+
+    settle(step)
     for _ in range(warmup):
-        fn()
+        step()
     torch.cuda.synchronize()
-    start = torch.cuda.Event(enable_timing=True)
-    end = torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(steps):
-        fn()
-    end.record()
+    names = list(kernels)
+    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(len(names) + 1)] for _ in range(steps)]
+    for i in range(steps):
+        marks[i][0].record()
+        for j, kname in enumerate(names):
+            kernels[kname]()
+            marks[i][j + 1].record()
     torch.cuda.synchronize()
-    return start.elapsed_time(end) / steps
+    per_step = [marks[i][0].elapsed_time(marks[i][-1]) for i in range(steps)]
+    mean_ms = marks[0][0].elapsed_time(marks[-1][-1]) / steps
+    per_kernel = {
+        kname: median([marks[i][j].elapsed_time(marks[i][j + 1]) for i in range(steps)]) for j, kname in enumerate(names)
+    }
+    return median(per_step), mean_ms, per_kernel
 
 
-def cpu_baseline(w, sample_tokens):
-    """The reference's CPU dense-equivalent path (to_dense + matmul, fp32) on the first sample_tokens tokens."""
+def cpu_baseline(w, tokens):
+    """The reference's CPU dense-equivalent path (to_dense + matmul, fp32): 3 warm-up + 5 timed runs, median."""
     import torch
 
     from oracle import block_sparse_oracle as O
     from pytorch_block_sparse_amd import workloads
 
-    blocks, data, x, dy = workloads.make_inputs(w, tokens=sample_tokens)
+    blocks, data, x, dy = workloads.make_inputs(w, tokens=tokens)
     X, Y = w.grid
     mask = O.mask_from_blocks(X, Y, blocks)
     idx = O.build_indices(mask)
@@ -87,29 +141,73 @@ def cpu_baseline(w, sample_tokens):
     xf, dyf = x.float(), dy.float()
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
-    O.linear_fwd_bwd_torch_fp32(xf, dyf, w_dense, mask_dense)  # warm-up
+    for _ in range(3):
+        O.linear_fwd_bwd_torch_fp32(xf, dyf, w_dense, mask_dense)
     times = []
-    t_all = time.perf_counter()
-    while len(times) < 5 and (len(times) < 2 or time.perf_counter() - t_all < 20.0):
+    for _ in range(5):
         t0 = time.perf_counter()
         O.linear_fwd_bwd_torch_fp32(xf, dyf, w_dense, mask_dense)
         times.append(time.perf_counter() - t0)
-    med = sorted(times)[len(times) // 2]
-    eff = 3 * 2.0 * sample_tokens * w.nnz * 1024 / med / 1e12
+    med = median(times)
+    eff = 3 * 2.0 * tokens * w.nnz * 1024 / med / 1e12
+    what = "all" if tokens == w.tokens else f"first {tokens} of"
     return {
         "value": eff,
         "unit": "TFLOP/s",
         "cores": cores,
         "kind": "port",
-        "sample": f"first {sample_tokens} of {w.tokens} tokens, same layer; torch CPU fp32 dense-equivalent "
-        f"fwd+dX+dW, median of {len(times)} runs ({med * 1e3:.1f} ms)",
+        "sample": f"{what} {w.tokens} tokens, same layer; torch CPU fp32 dense-equivalent fwd+dX+dW, "
+        f"3 warm-up + 5 timed runs, median {med * 1e3:.1f} ms",
     }
 
 
-ROBERTA_WORKLOAD = "c5_roberta_base_mlm_fp32"
+def measure_layer(w, tokens, steps, warmup, dense=True):
+    """Times the GEMMs of one BlockSparseLinear workload; returns the figures the JSON line is built from."""
+    import torch
+
+    from pytorch_block_sparse_amd import BlockSparseMatrix, workloads
+
+    dev = torch.device("cuda:0")
+    blocks, data, x, dy = workloads.make_inputs(w, tokens=tokens)
+    m = BlockSparseMatrix.zeros((w.out_features, w.in_features), blocks=blocks, device="cpu", dtype=w.dtype)
+    with torch.no_grad():
+        m.data.copy_(data)
+    m = m.to(dev)
+    xd, dyd = x.to(dev), dy.to(dev)
+    torch.cuda.synchronize()
+    kernels = {"fwd": lambda: m.reverse_matmul(xd, True)}
+    if w.passes != "fwd":
+        kernels["dx"] = lambda: m.reverse_matmul(dyd, False)
+        kernels["dw"] = lambda: m.matmul_with_output_sparse_support(dyd, xd)
+    ms_step, ms_mean, per_kernel = time_steps(kernels, steps, warmup)
+    dname = "bf16" if w.dtype == torch.bfloat16 else "f32"
+    flops_gemm = 2.0 * tokens * w.nnz * 1024
+    res = {
+        "dtype": dname,
+        "tokens": tokens,
+        "n_gemms": len(kernels),
+        "flops_gemm": flops_gemm,
+        "ms_per_step": ms_step,
+        "ms_per_step_mean": ms_mean,
+        "kernel_ms": per_kernel,
+        "value": len(kernels) * flops_gemm / (ms_step * 1e-3) / 1e12,
+    }
+    if dense:
+        wd = m.to_dense()
+        dk = {"fwd": lambda: xd @ wd.t()}
+        if w.passes != "fwd":
+            dk["dx"] = lambda: dyd @ wd
+            dk["dw"] = lambda: dyd.t() @ xd
+        ms_dense, _, _ = time_steps(dk, steps, warmup)
+        res["dense"] = {
+            "ms_per_step": ms_dense,
+            "dense_tflops": len(dk) * 2.0 * tokens * w.in_features * w.out_features / (ms_dense * 1e-3) / 1e12,
+            "speedup_sparse_vs_dense": ms_dense / ms_step,
+        }
+    return res
 
 
-def run_roberta(args):
+def measure_roberta(steps, warmup):
     """One MLM training step (forward + backward + AdamW, fp32) of a 12-layer RoBERTa-base-shaped encoder
     with random weights, batch 32 x 512 random token ids, once with dense linear layers and once with
     attention.output.dense, intermediate.dense and output.dense of every layer patched to block-sparse
@@ -117,9 +215,8 @@ def run_roberta(args):
     import torch
     from transformers import RobertaConfig, RobertaForMaskedLM
 
-    from pytorch_block_sparse_amd import BlockSparseLinear, BlockSparseModelPatcher, native
+    from pytorch_block_sparse_amd import BlockSparseLinear, BlockSparseModelPatcher
 
-    native.load()
     dev = torch.device("cuda:0")
     batch, seq = 32, 512
     cfg = RobertaConfig(vocab_size=50265, hidden_size=768, num_hidden_layers=12, num_attention_heads=12,
@@ -138,12 +235,16 @@ def run_roberta(args):
         model = model.to(dev)
         n_layers = 0
         if sparse:
+            import contextlib
+            import io
+
             mp = BlockSparseModelPatcher()
             for pat in (r"roberta\.encoder\.layer\.[0-9]+\.attention\.output\.dense",
                         r"roberta\.encoder\.layer\.[0-9]+\.intermediate\.dense",
                         r"roberta\.encoder\.layer\.[0-9]+\.output\.dense"):
                 mp.add_pattern(pat, {"density": 0.5})
-            mp.patch_model(model)
+            with contextlib.redirect_stdout(io.StringIO()):   # the patcher prints one line per layer
+                mp.patch_model(model)
             n_layers = sum(isinstance(m, BlockSparseLinear) for m in model.modules())
         return model, n_dense, sum(p.numel() for p in model.parameters()), n_layers
 
@@ -157,16 +258,16 @@ def run_roberta(args):
             opt.zero_grad(set_to_none=True)
             return loss
 
-        for _ in range(args.warmup):
+        for _ in range(warmup):
             one()
         torch.cuda.synchronize()
-        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record()
-        for _ in range(args.steps):
+        marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+        marks[0].record()
+        for i in range(steps):
             loss = one()
-        end.record()
+            marks[i + 1].record()
         torch.cuda.synchronize()
-        return start.elapsed_time(end) / args.steps, float(loss)
+        return median([marks[i].elapsed_time(marks[i + 1]) for i in range(steps)]), float(loss.detach())
 
     model, n_dense, _, _ = build(False)
     ms_dense, loss_dense = time_model(model)
@@ -174,26 +275,48 @@ def run_roberta(args):
     torch.cuda.empty_cache()
     model, _, n_sparse, n_layers = build(True)
     ms_sparse, loss_sparse = time_model(model)
-    tokens = batch * seq
+    del model
+    torch.cuda.empty_cache()
+    return {
+        "batch": batch, "seq_len": seq, "patched_layers": n_layers, "steps": steps, "warmup": warmup,
+        "dense_model": {"ms_per_step": ms_dense, "parameters": n_dense, "loss": loss_dense},
+        "sparse_model": {"ms_per_step": ms_sparse, "parameters": n_sparse, "loss": loss_sparse},
+        "tokens_per_s": batch * seq / (ms_sparse * 1e-3),
+        "speedup_sparse_vs_dense": ms_dense / ms_sparse,
+    }
+
+
+def roberta_line(args):
+    r = measure_roberta(args.steps, args.warmup)
     print(json.dumps({
         "metric": "MLM training step of a RoBERTa-base-shaped encoder, 36 linear layers block-sparse at density 0.5",
-        "value": tokens / (ms_sparse * 1e-3),
+        "value": r["tokens_per_s"],
         "unit": "tokens/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": ms_sparse,
+        "ms_per_step": r["sparse_model"]["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": ROBERTA_WORKLOAD, "layers": 12, "hidden": 768, "ffn": 3072, "vocab": 50265,
-                   "batch": batch, "seq_len": seq, "density": 0.5, "patched_layers": n_layers},
-        "dense_model": {"ms_per_step": ms_dense, "parameters": n_dense, "loss": loss_dense},
-        "sparse_model": {"ms_per_step": ms_sparse, "parameters": n_sparse, "loss": loss_sparse},
-        "speedup_sparse_vs_dense": ms_dense / ms_sparse,
+                   "batch": r["batch"], "seq_len": r["seq_len"], "density": 0.5, "patched_layers": r["patched_layers"]},
+        "dense_model": r["dense_model"],
+        "sparse_model": r["sparse_model"],
+        "speedup_sparse_vs_dense": r["speedup_sparse_vs_dense"],
     }))
+
+
+def kernel_label(w, tokens, which):
+    dname = "bf16" if w.dtype.itemsize == 2 else "f32"
+    if which == "dw":
+        return ("sdd_bf16_kernel" if dname == "bf16" else "sdd_kernel") + " (+ sdd_reduce_kernel)"
+    n, k, trans = (w.out_features, w.in_features, 0) if which == "fwd" else (w.in_features, w.out_features, 1)
+    # the library picks the wide-tile kernel for bf16 when there are at least 256 tiles of 128 tokens x 512 columns
+    wide = dname == "bf16" and k % 64 == 0 and ((tokens + 127) // 128) * ((n // 32 + 15) // 16) >= 256
+    return ("dds16_kernel" if wide else "dds_kernel") + f"<TRANS={trans}>"
 
 
 def main():
@@ -201,95 +324,39 @@ def main():
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only; --gpus must be 1", file=sys.stderr)
         sys.exit(2)
-    if args.workload == ROBERTA_WORKLOAD:
-        run_roberta(args)
-        return
     import torch
 
-    from pytorch_block_sparse_amd import BlockSparseMatrix, native, workloads
+    from pytorch_block_sparse_amd import native, workloads
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(3)
     native.load()  # fail loudly if the HIP library is not built
-    dev = torch.device("cuda:0")
+    if args.workload == ROBERTA_WORKLOAD:
+        roberta_line(args)
+        return
     w = workloads.WORKLOADS[args.workload]
     tokens = args.tokens or w.tokens
-    blocks, data, x, dy = workloads.make_inputs(w, tokens=tokens)
-    m = BlockSparseMatrix.zeros((w.out_features, w.in_features), blocks=blocks, device="cpu", dtype=w.dtype)
-    with torch.no_grad():
-        m.data.copy_(data)
-    m = m.to(dev)
-    xd, dyd = x.to(dev), dy.to(dev)
-    torch.cuda.synchronize()
-
-    def fwd():
-        return m.reverse_matmul(xd, True)
-
-    def dx():
-        return m.reverse_matmul(dyd, False)
-
-    def dw():
-        return m.matmul_with_output_sparse_support(dyd, xd)
-
-    if w.passes == "fwd":
-        kernels = {"fwd": fwd}
-    else:
-        kernels = {"fwd": fwd, "dx": dx, "dw": dw}
-
-    def step():
-        for f in kernels.values():
-            f()
-
-    # The timed region is exactly `steps` steps.  Inside it an event is recorded after every kernel, so
-    # that the per-kernel durations are those of the launches of the timed steps themselves (the same
-    # launches a rocprofv3 kernel trace of this command averages), not of a kernel repeated on its own.
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    names = list(kernels)
-    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(len(names) + 1)] for _ in range(args.steps)]
-    for i in range(args.steps):
-        marks[i][0].record()
-        for j, kname in enumerate(names):
-            kernels[kname]()
-            marks[i][j + 1].record()
-    torch.cuda.synchronize()
-    ms_step = marks[0][0].elapsed_time(marks[-1][-1]) / args.steps
-    per_kernel = {
-        kname: sum(marks[i][j].elapsed_time(marks[i][j + 1]) for i in range(args.steps)) / args.steps
-        for j, kname in enumerate(names)
-    }
-
-    dname = "bf16" if w.dtype == torch.bfloat16 else "f32"
-    flops_gemm = 2.0 * tokens * w.nnz * 1024
-    n_gemms = len(kernels)
-    value = n_gemms * flops_gemm / (ms_step * 1e-3) / 1e12
+    r = measure_layer(w, tokens, args.steps, args.warmup, dense=not args.no_dense)
+    dname, per_kernel, flops_gemm = r["dtype"], r["kernel_ms"], r["flops_gemm"]
     dom = max(per_kernel, key=per_kernel.get)
     achieved = flops_gemm / (per_kernel[dom] * 1e-3) / 1e12
-    sdd = "sdd_bf16_kernel" if dname == "bf16" else "sdd_kernel"
-
-    def dds_name(n, k, trans):
-        # the library picks the wide-tile kernel for bf16 when there are at least 256 tiles of 128 tokens x 512 columns
-        wide = dname == "bf16" and k % 64 == 0 and ((tokens + 127) // 128) * ((n // 32 + 15) // 16) >= 256
-        return ("dds16_kernel" if wide else "dds_kernel") + f"<TRANS={trans}>"
-
-    kernel_names = {
-        "fwd": dds_name(w.out_features, w.in_features, 0),
-        "dx": dds_name(w.in_features, w.out_features, 1),
-        "dw": sdd + " (+ sdd_reduce_kernel)",
-    }
-    traffic = MEASURED_TRAFFIC.get((w.name, tokens), {}).get(dom)
+    # which roofline bounds the kernel: time at the matrix peak against time at the HBM peak for the algorithmic bytes
+    e = 2 if dname == "bf16" else 4
+    alg_bytes = e * (tokens * w.in_features + tokens * w.out_features + w.nnz * 1024)
+    t_mfma = flops_gemm / (PEAK_TFLOPS[dname] * 1e12)
+    t_hbm = alg_bytes / (HBM_TBPS * 1e12)
 
     out = {
         "metric": BASELINE_METRIC if w.name == BASELINE_WORKLOAD and tokens == w.tokens
         else f"effective TFLOP/s of the block-sparse GEMMs ({w.passes}) of {w.name} at {tokens} tokens",
-        "value": value,
+        "value": r["value"],
         "unit": "TFLOP/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": ms_step,
+        "ms_per_step": r["ms_per_step"],
+        "ms_per_step_mean": r["ms_per_step_mean"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -305,54 +372,65 @@ def main():
             "pattern": w.pattern,
             "passes": w.passes,
         },
-        "pct_of_mfma_peak": 100.0 * value / PEAK_TFLOPS[dname],
+        "pct_of_mfma_peak": 100.0 * r["value"] / PEAK_TFLOPS[dname],
         "kernel_ms": per_kernel,
         "kernel_eff_tflops": {k: flops_gemm / (v * 1e-3) / 1e12 for k, v in per_kernel.items()},
         "roofline": {
-            "bound": "mfma",
-            "kernel": kernel_names[dom],
+            "bound": "mfma" if t_mfma >= t_hbm else "hbm",
+            "kernel": kernel_label(w, tokens, dom),
             "achieved": achieved,
             "peak": PEAK_TFLOPS[dname],
             "unit": "TFLOP/s",
             "frac": achieved / PEAK_TFLOPS[dname],
-            "traffic": traffic,
+            "traffic": measured_traffic(w.name, tokens, dom),
             "traffic_unit": "bytes per launch",
             "flops_per_launch": flops_gemm,
+            "algorithmic_bytes_per_launch": alg_bytes,
         },
     }
-
-    if not args.no_dense:
-        wd = m.to_dense()
-        dense = {
-            "fwd": lambda: xd @ wd.t(),
-            "dx": lambda: dyd @ wd,
-            "dw": lambda: dyd.t() @ xd,
-        }
-        if w.passes == "fwd":
-            dense = {"fwd": dense["fwd"]}
-
-        def dense_step():
-            for f in dense.values():
-                f()
-
-        ms_dense = time_gpu(dense_step, args.steps, args.warmup)
-        out["dense_hipblaslt"] = {
-            "ms_per_step": ms_dense,
-            "dense_tflops": n_gemms * 2.0 * tokens * w.in_features * w.out_features / (ms_dense * 1e-3) / 1e12,
-            "speedup_sparse_vs_dense": ms_dense / ms_step,
-        }
-        del wd
+    if "dense" in r:
+        out["dense_hipblaslt"] = r["dense"]
 
     if args.copy_calibration:
-        src = torch.empty(1 << 28, dtype=torch.uint8, device=dev).fill_(1)
+        src = torch.empty(1 << 28, dtype=torch.uint8, device="cuda:0").fill_(1)
         dst = torch.empty_like(src)
         for _ in range(3):
             dst.copy_(src)
         torch.cuda.synchronize()
         out["copy_calibration_bytes"] = 1 << 28
 
+    if not args.no_others and w.name == BASELINE_WORKLOAD and tokens == w.tokens:
+        others = {}
+        for name in OTHER_LAYER_WORKLOADS:
+            ow = workloads.WORKLOADS[name]
+            o = measure_layer(ow, ow.tokens, 30, 10, dense=not args.no_dense)
+            peak = PEAK_TFLOPS[o["dtype"]]
+            slow = max(o["kernel_ms"], key=o["kernel_ms"].get)
+            others[name] = {
+                "ms_per_step": o["ms_per_step"],
+                "value": o["value"],
+                "unit": "TFLOP/s",
+                "frac": o["flops_gemm"] / (o["kernel_ms"][slow] * 1e-3) / 1e12 / peak,   # slowest kernel against the fp32 peak
+                "pct_of_mfma_peak": 100.0 * o["value"] / peak,
+                "kernel_ms": o["kernel_ms"],
+                "vs_dense": o["dense"]["speedup_sparse_vs_dense"] if "dense" in o else None,
+            }
+        try:
+            rb = measure_roberta(5, 2)
+            others[ROBERTA_WORKLOAD] = {
+                "ms_per_step": rb["sparse_model"]["ms_per_step"],
+                "value": rb["tokens_per_s"],
+                "unit": "tokens/s",
+                "dense_ms_per_step": rb["dense_model"]["ms_per_step"],
+                "vs_dense": rb["speedup_sparse_vs_dense"],
+                "patched_layers": rb["patched_layers"],
+            }
+        except ImportError as exc:   # transformers missing: the layer workloads above still stand
+            others[ROBERTA_WORKLOAD] = {"skipped": str(exc)}
+        out["other_configs"] = others
+
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(w, min(args.cpu_sample_tokens, tokens))
+        out["cpu_baseline"] = cpu_baseline(w, args.cpu_sample_tokens or tokens)
     print(json.dumps(out))
 
 
