@@ -54,10 +54,6 @@ static int launch_dds(DdsArgs g, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
-#ifndef PBS_SHAPE3_FACTOR
-#define PBS_SHAPE3_FACTOR 0.8
-#endif
-
 // ---- wide-tile persistent bf16 kernel ----
 // The plan buffer holds the narrow plan first, then (when k is a multiple of 64) the wide one.
 static inline size_t narrow_plan_bytes(int n, int k) {
@@ -141,7 +137,7 @@ static int dispatch_dds(const DdsArgs& g, hipStream_t stream) {
         (long long)((g.M + 127) / 128) * g.n_groups * 2,
         (long long)((g.M + 255) / 256) * g.n_groups,
     };
-    const double area[4] = {2048.0, 1024.0 * 1.04, 512.0 * 1.10, 2048.0 * PBS_SHAPE3_FACTOR};
+    const double area[4] = {2048.0, 1024.0 * 1.04, 512.0 * 1.10, 2048.0 * 0.8};
     double cost[4];
     for (int c = 0; c < NSHAPES; ++c) cost[c] = (double)((tiles[c] + 255) / 256) * area[c];
     int order[4] = {0, 1, 2, 3};
@@ -176,7 +172,7 @@ struct SddShapeF32 {
     static constexpr int SR = 8, SC = 8, QW = 8, NW = 8, TC = 16;
 };
 struct SddShapeBf16 {
-    static constexpr int SR = 16, SC = 16, QW = 10, TC = 32, NS = 2;
+    static constexpr int SR = 16, SC = 16, QW = 10, TC = 32, NS = 2, NW = 8;
 };
 
 struct SddPlan {
@@ -233,10 +229,10 @@ static int launch_sdd(SddArgs a, int dtype, void* workspace, size_t workspace_by
         hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)wgs)), dim3(C::NT), C::LDS_BYTES, stream, a);
     } else {
         using S = SddShapeBf16;
-        using C = SddBf16Cfg<S::QW, S::TC, S::NS>;
+        using C = SddBf16Cfg<S::QW, S::TC, S::NS, S::NW>;
         static_assert(C::TC == S::TC && C::SR == S::SR && C::SC == S::SC, "plan and kernel must agree");
         static std::atomic<uint64_t> done{0};
-        auto kernel = sdd_bf16_kernel<S::QW, S::TC, S::NS>;
+        auto kernel = sdd_bf16_kernel<S::QW, S::TC, S::NS, S::NW>;
         if (int rc = raise_lds_limit(kernel, C::LDS_BYTES, done)) return rc;
         hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)wgs)), dim3(C::NT), C::LDS_BYTES, stream, a);
     }

@@ -24,9 +24,9 @@
 
 namespace pbs {
 
-template <int QW, int TC_, int NS_>
+template <int QW, int TC_, int NS_, int NW_ = 8>
 struct SddBf16Cfg {
-    static constexpr int SR = 16, SC = 16, NW = 8, NT = NW * 64;
+    static constexpr int SR = 16, SC = 16, NW = NW_, NT = NW * 64;
     static constexpr int TC = TC_;                           // tokens per chunk (16 or 32)
     static constexpr int NS = NS_;                           // chunk buffers: NS - 1 chunks of loads in flight
     static constexpr int ROW_BYTES = 1024;                   // one token row of a panel: 16 blocks x 32 x 2 B
@@ -38,6 +38,7 @@ struct SddBf16Cfg {
     static constexpr int ROWS_PER_WAVE = TC / NW;            // token rows of each panel a wave copies per chunk
     static_assert(TC_ == 16 || TC_ == 32, "one or two 16-token matrix steps per chunk");
     static_assert(NS_ >= 2 && NS_ <= 4, "chunk buffers");
+    static_assert(QW >= ROWS_PER_WAVE, "a wave issues its token rows between its block products");
 };
 
 // The rectangle's rows, columns and block list, built by all threads of the workgroup (NT threads, of
@@ -234,9 +235,9 @@ static __device__ __forceinline__ void sdd_bf16_prologue(const SddArgs& a, int t
     __syncthreads();
 }
 
-template <int QW, int TC_, int NS_>
-__global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
-    using C = SddBf16Cfg<QW, TC_, NS_>;
+template <int QW, int TC_, int NS_, int NW_ = 8>
+__global__ __launch_bounds__(NW_ * 64) void sdd_bf16_kernel(SddArgs a) {
+    using C = SddBf16Cfg<QW, TC_, NS_, NW_>;
     constexpr int NS = C::NS;
     constexpr int SR = C::SR, SC = C::SC, NW = C::NW, TC = C::TC;
 
@@ -285,31 +286,49 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
     const int x_cid = x_unit >= 0 ? x_unit * 2 + ((pc >> 2) & 1) : -1;
     const unsigned x_voff = (x_cid >= 0 && x_cid < nblk_c) ? (unsigned)(x_cid * 64 + (pc & 3) * 16) : 0u;
     const size_t g_row_bytes = (size_t)a.N * 2, x_row_bytes = (size_t)a.K * 2;
-    const unsigned char* g_col = G;
-    const unsigned char* x_col = X;
 
-    // returns the number of DMA instructions issued (wave-uniform)
-    // token row number k of this wave's ROWS_PER_WAVE, both panels, of chunk ci; returns the DMA count
-    auto issue_row = [&](int ci, int k) -> int {
-        const int buf = ci % NS;
-        const int tl = wave + k * NW;
-        const int t = t_begin + ci * TC + tl;
+    // DMA issue state: chunks are issued in order; the addresses of the chunk being issued are kept and
+    // advanced by constant strides (a 64-bit multiply per row and panel cost more scalar instructions per
+    // chunk than all the rest of the chunk's bookkeeping).
+    const size_t g_kstep = (size_t)NW * g_row_bytes, x_kstep = (size_t)NW * x_row_bytes;   // between this wave's rows
+    const size_t g_cstep = (size_t)TC * g_row_bytes, x_cstep = (size_t)TC * x_row_bytes;   // between chunks
+    int iss_t = 0;                       // token of this wave's first row in the chunk being issued
+    unsigned iss_stage = 0;              // LDS address of that row in the chunk's buffer
+    const unsigned char* iss_g = G;      // global address of that row, G panel
+    const unsigned char* iss_x = X;
+    auto issue_reset = [&]() {
+        iss_t = t_begin + wave;
+        iss_stage = lds0 + wave * C::ROW_BYTES;
+        iss_g = uniform_ptr(G + (size_t)iss_t * g_row_bytes);
+        iss_x = uniform_ptr(X + (size_t)iss_t * x_row_bytes);
+    };
+    // token row number k of this wave's ROWS_PER_WAVE, both panels, of the chunk being issued; returns the DMA count
+    auto issue_row = [&](int k) -> int {
+        const int t = iss_t + k * NW;
+        const unsigned stage = iss_stage + k * NW * C::ROW_BYTES;
         if (t < t_end) {
-            const unsigned stage = lds0 + buf * C::STAGE_BYTES + tl * C::ROW_BYTES;
-            dma16(stage, uniform_ptr(g_col + (size_t)t * g_row_bytes), g_voff);
-            dma16(stage + C::PANEL_BYTES, uniform_ptr(x_col + (size_t)t * x_row_bytes), x_voff);
+            dma16(stage, iss_g + k * g_kstep, g_voff);
+            dma16(stage + C::PANEL_BYTES, iss_x + k * x_kstep, x_voff);
             return 2;
         }
         // tokens past the end contribute nothing
-        unsigned char* p = smem + buf * C::STAGE_BYTES + tl * C::ROW_BYTES + lane * 16;
+        unsigned char* p = smem + (stage - lds0) + lane * 16;
         *reinterpret_cast<uint4*>(p) = make_uint4(0, 0, 0, 0);
         *reinterpret_cast<uint4*>(p + C::PANEL_BYTES) = make_uint4(0, 0, 0, 0);
         return 0;
     };
-    auto issue_chunk = [&](int ci) -> int {
+    auto issue_next = [&]() {   // the next chunk goes to the next buffer
+        iss_t += TC;
+        iss_g += g_cstep;
+        iss_x += x_cstep;
+        iss_stage += C::STAGE_BYTES;
+        if (iss_stage >= lds0 + NS * C::STAGE_BYTES) iss_stage -= NS * C::STAGE_BYTES;
+    };
+    auto issue_chunk = [&]() -> int {
         int n = 0;
 #pragma unroll
-        for (int k = 0; k < C::ROWS_PER_WAVE; ++k) n += issue_row(ci, k);
+        for (int k = 0; k < C::ROWS_PER_WAVE; ++k) n += issue_row(k);
+        issue_next();
         return n;
     };
 
@@ -362,25 +381,50 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
                 f[u] = make_uint4(lo.x, lo.y, hi.x, hi.y);
             }
         };
-        auto compute_chunk = [&](int ci) {
+        // products of chunk ci; the DMA of the next chunk to issue (if do_issue) goes between them, one token row
+        // of both panels after each of the first blocks, so that the texture path works while the matrix
+        // cores do (issued in one go ahead of the products, the copy instructions hold the wave for as long
+        // as the texture path needs for the whole chunk, and the products only start after that).
+        // Returns the number of DMA instructions issued.
+        auto compute_chunk = [&](int ci, bool do_issue) -> int {
             const unsigned char* stage = smem + (ci % NS) * C::STAGE_BYTES;
-            uint4 fb[NU];
-            int cur_rl = -1;
+            int n_dma = 0;
+            // The fragments of block q + 1 are fetched before the products of block q are issued, so that the
+            // LDS round trip of one block runs under the matrix instructions of the one before it (fetched
+            // right before their own products, the eight or so round trips of a chunk added up to twice the
+            // matrix time).  The loop is unrolled: the two fragment sets alternate by name, not by copying.
+            uint4 fa[2][NU], fb[2][NU];
+            if (w_n > 0) {
+                load_frag(fb[0], stage + b_off[0]);
+                load_frag(fa[0], stage + a_off[0]);
+            }
 #pragma unroll
             for (int q = 0; q < QW; ++q) {
+                if (q >= w_n && q < C::ROWS_PER_WAVE && do_issue) n_dma += issue_row(q);   // fewer blocks than rows to copy
                 if (q < w_n) {
-                    if (rl_of[q] != cur_rl) {
-                        load_frag(fb, stage + b_off[q]);
-                        cur_rl = rl_of[q];
+                    constexpr int cur = 0, nxt = 1;
+                    uint4(&fa_c)[NU] = fa[(q & 1) ? nxt : cur];
+                    uint4(&fb_c)[NU] = fb[(q & 1) ? nxt : cur];
+                    uint4(&fa_n)[NU] = fa[(q & 1) ? cur : nxt];
+                    uint4(&fb_n)[NU] = fb[(q & 1) ? cur : nxt];
+                    if (q + 1 < QW && q + 1 < w_n) {
+                        load_frag(fa_n, stage + a_off[q + 1]);
+                        if (rl_of[q + 1] != rl_of[q]) {
+                            load_frag(fb_n, stage + b_off[q + 1]);
+                        } else {
+#pragma unroll
+                            for (int u = 0; u < NU; ++u) fb_n[u] = fb_c[u];
+                        }
                     }
-                    uint4 fa[NU];
-                    load_frag(fa, stage + a_off[q]);
 #pragma unroll
                     for (int u = 0; u < NU; ++u)
-                        acc[q] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa[u]),
-                                                                         __builtin_bit_cast(bf16x8, fb[u]), acc[q], 0, 0, 0);
+                        acc[q] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa_c[u]),
+                                                                         __builtin_bit_cast(bf16x8, fb_c[u]), acc[q], 0, 0, 0);
+                    if (q < C::ROWS_PER_WAVE && do_issue) n_dma += issue_row(q);
                 }
             }
+            if (do_issue) issue_next();
+            return n_dma;
         };
 
         if (nchunks > 0) {
@@ -388,20 +432,25 @@ __global__ __launch_bounds__(512) void sdd_bf16_kernel(SddArgs a) {
             int pend[NS];
 #pragma unroll
             for (int k = 0; k < NS; ++k) pend[k] = 0;
+            issue_reset();
 #pragma unroll
             for (int k = 0; k < NS - 1; ++k)
-                if (k < nchunks) pend[k] = issue_chunk(k);
+                if (k < nchunks) pend[k] = issue_chunk();
             for (int ci = 0; ci < nchunks; ++ci) {
-                int later = 0;
-#pragma unroll
-                for (int k = 1; k < NS; ++k) later += pend[k];
                 // chunk ci has landed for every wave, and every wave is done reading chunk ci - 1
-                wait_dma_and_barrier(later);
+                if constexpr (NS == 2) {
+                    drain_barrier();   // with two buffers nothing younger than chunk ci is in flight
+                } else {
+                    int later = 0;
+#pragma unroll
+                    for (int k = 1; k < NS; ++k) later += pend[k];
+                    wait_dma_and_barrier(later);
+                }
 #pragma unroll
                 for (int k = 0; k + 1 < NS; ++k) pend[k] = pend[k + 1];
                 pend[NS - 1] = 0;
-                if (ci + NS - 1 < nchunks) pend[NS - 2] = issue_chunk(ci + NS - 1);   // into the buffer of chunk ci - 1
-                compute_chunk(ci);
+                // chunk ci + NS - 1 goes into the buffer of chunk ci - 1, which every wave has left
+                pend[NS - 2] = compute_chunk(ci, ci + NS - 1 < nchunks);
             }
             lds_barrier();   // the next pass refills the buffers
         }
