@@ -58,10 +58,12 @@ static inline size_t dds_plan_group_ints(int KB) { return ((size_t)KB + 2) * DDS
 // per-column block counts are very uneven (largest > 2x the mean) the columns are ranked by count
 // and dealt to the half-groups of 4 in serpentine order, so every tile gets about the same number
 // of blocks: a tile of a few heavy columns would otherwise run long after all others are done.
+// A group may also be given fewer than 8 columns (width), which leaves places empty: more, lighter
+// tiles, for launches that would otherwise leave CUs without one.
 // slots[8g + j] = block column in place j of group g, or -1.  One workgroup.
 constexpr int DDS_BALANCE_MAX_COLS = 4096;
 __global__ __launch_bounds__(256) void dds_slots_kernel(const int32_t* __restrict__ ptr, int nblk_n, int n_groups,
-                                                        int* slots) {
+                                                        int width, int* slots) {
     constexpr int NT = 256;
     __shared__ int s_cnt[DDS_BALANCE_MAX_COLS];
     __shared__ int s_slot[DDS_BALANCE_MAX_COLS + DDS_NB];
@@ -85,7 +87,15 @@ __global__ __launch_bounds__(256) void dds_slots_kernel(const int32_t* __restric
         skewed = (long long)s_max * nblk_n > 2ll * s_sum;
     }
     if (!skewed) {
-        for (int i = tid; i < total; i += NT) slots[i] = i < nblk_n ? i : -1;
+        // group g holds columns g * width .. + width - 1; with fewer than 8 they alternate between the two
+        // halves of the group's places, so that tiles of 4 places and the column halves of the waves get
+        // equal shares
+        for (int i = tid; i < total; i += NT) {
+            const int j = i % DDS_NB;
+            const int l = width == DDS_NB ? j : (j < 4 ? 2 * j : 2 * (j - 4) + 1);
+            const int c = (i / DDS_NB) * width + l;
+            slots[i] = (l < width && c < nblk_n) ? c : -1;
+        }
         return;
     }
     for (int i = tid; i < total; i += NT) s_slot[i] = -1;

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <cmath>
 #include <mutex>
 
 #include "pbs_common.h"
@@ -56,18 +57,43 @@ static int launch_dds(DdsArgs g, hipStream_t stream) {
 
 // ---- wide-tile persistent bf16 kernel ----
 // The plan buffer holds the narrow plan first, then (when k is a multiple of 64) the wide one.
-static inline size_t narrow_plan_bytes(int n, int k) {
-    const size_t groups = ((size_t)(n / 32) + DDS_NB - 1) / DDS_NB;
-    return groups * dds_plan_group_ints(k / 32) * sizeof(int);
+// The narrow plan exists in four versions that differ in how many block columns of the result a
+// group of 8 places holds (8, 7, 6 or 5; the other places stay empty): one workgroup runs per CU, so a
+// launch whose tiles number 192 leaves a quarter of the chip idle, while the same columns in groups
+// of 6 make 256 tiles of three quarters the work each.  Which version a launch uses depends on the
+// token count, which is not known when the plan is built.
+constexpr int DDS_NWIDTHS = 4;
+constexpr int DDS_WIDTHS[DDS_NWIDTHS] = {8, 7, 6, 5};
+static inline size_t narrow_groups(int n, int wi) { return ((size_t)(n / 32) + DDS_WIDTHS[wi] - 1) / DDS_WIDTHS[wi]; }
+static inline size_t narrow_plan_bytes_w(int n, int k, int wi) {
+    return narrow_groups(n, wi) * dds_plan_group_ints(k / 32) * sizeof(int);
 }
-static inline size_t slot_table_bytes(int n) {   // behind the plans: the block column in every place of every group
-    const size_t groups = ((size_t)(n / 32) + DDS_NB - 1) / DDS_NB;
-    return ((groups * DDS_NB * sizeof(int)) + 63) / 64 * 64;
+static inline size_t slot_table_bytes_w(int n, int wi) {   // the block column in every place of every group
+    return ((narrow_groups(n, wi) * DDS_NB * sizeof(int)) + 63) / 64 * 64;
 }
+// Plan buffer: [narrow plan, 8 columns per group][wide plan][slot table, 8][narrow 7][slots 7][narrow 6][slots 6]
+// [narrow 5][slots 5].
+static inline size_t narrow_plan_bytes(int n, int k) { return narrow_plan_bytes_w(n, k, 0); }
+static inline size_t slot_table_bytes(int n) { return slot_table_bytes_w(n, 0); }
 static inline size_t wide_plan_bytes(int n, int k) {
     if (k % 64) return 0;
     const size_t groups = ((size_t)(n / 32) + D16_NB - 1) / D16_NB;
     return (groups * dds16_plan_group_ints(k / 32) + D16_SEQ_INTS) * sizeof(int);
+}
+
+static inline size_t narrow_plan_offset(int n, int k, int wi) {
+    if (wi == 0) return 0;
+    size_t off = narrow_plan_bytes(n, k) + wide_plan_bytes(n, k) + slot_table_bytes(n);
+    for (int i = 1; i < wi; ++i) off += narrow_plan_bytes_w(n, k, i) + slot_table_bytes_w(n, i);
+    return off;
+}
+static inline size_t slot_table_offset(int n, int k, int wi) {
+    if (wi == 0) return narrow_plan_bytes(n, k) + wide_plan_bytes(n, k);
+    return narrow_plan_offset(n, k, wi) + narrow_plan_bytes_w(n, k, wi);
+}
+static inline size_t all_plan_bytes(int n, int k) {
+    return narrow_plan_offset(n, k, DDS_NWIDTHS - 1) + narrow_plan_bytes_w(n, k, DDS_NWIDTHS - 1) +
+           slot_table_bytes_w(n, DDS_NWIDTHS - 1);
 }
 
 constexpr int D16_TM = 2, D16_RS = 3, D16_RB = 32, D16_NP = 4;
@@ -130,57 +156,82 @@ static int dispatch_dds(const DdsArgs& g, hipStream_t stream) {
     // shapes: 0 = 256 x 8 (4 token slices x 2 column halves), 1 = 128 x 8, 2 = 128 x 4,
     //         3 = 256 x 8 with 8 token slices (every wave has all 8 columns; fp32 only: 8 accumulators of fp32
     //             fragments fit the registers, and balanced waves are worth more than the larger fragments cost)
+    // widths: 8, 7, 6 or 5 of a tile's 8 (4) places hold a block column.  A tile's time falls with the columns it
+    //         holds, though not in proportion (its panel traffic and per-step overhead stay); bf16 tiles are
+    //         bound by their operand stream rather than by the matrix cores and gain less.
     constexpr int NSHAPES = sizeof(T) == 4 ? 4 : 3;
-    const long long tiles[4] = {
-        (long long)((g.M + 255) / 256) * g.n_groups,
-        (long long)((g.M + 127) / 128) * g.n_groups,
-        (long long)((g.M + 127) / 128) * g.n_groups * 2,
-        (long long)((g.M + 255) / 256) * g.n_groups,
-    };
+    constexpr int NCAND = NSHAPES * DDS_NWIDTHS;
     const double area[4] = {2048.0, 1024.0 * 1.04, 512.0 * 1.10, 2048.0 * 0.8};
-    double cost[4];
-    for (int c = 0; c < NSHAPES; ++c) cost[c] = (double)((tiles[c] + 255) / 256) * area[c];
-    int order[4] = {0, 1, 2, 3};
-    for (int i = 0; i < NSHAPES; ++i)
-        for (int j = i + 1; j < NSHAPES; ++j)
+    const double fixed = sizeof(T) == 4 ? 0.15 : 0.35;   // share of a tile's time that does not depend on its columns
+    double cost[NCAND];
+    int order[NCAND];
+    for (int wi = 0; wi < DDS_NWIDTHS; ++wi) {
+        const long long groups = (long long)narrow_groups(g.N, wi);
+        // of the widths that give the same number of groups only the narrowest (most even) is tried
+        const bool useful = wi == 0 || (groups > (long long)narrow_groups(g.N, 0) &&
+                                        (wi == DDS_NWIDTHS - 1 || groups != (long long)narrow_groups(g.N, wi + 1)));
+        const long long tiles[4] = {
+            (long long)((g.M + 255) / 256) * groups,
+            (long long)((g.M + 127) / 128) * groups,
+            (long long)((g.M + 127) / 128) * groups * 2,
+            (long long)((g.M + 255) / 256) * groups,
+        };
+        for (int c = 0; c < NSHAPES; ++c) {
+            const int i = wi * NSHAPES + c;
+            order[i] = i;
+            cost[i] = useful ? (double)((tiles[c] + 255) / 256) * area[c] * (fixed + (1.0 - fixed) * DDS_WIDTHS[wi] / 8.0) * (1.0 + 0.01 * wi)
+                             : 1e300;
+        }
+    }
+    for (int i = 0; i < NCAND; ++i)
+        for (int j = i + 1; j < NCAND; ++j)
             if (cost[order[j]] < cost[order[i]]) {
                 const int t = order[i];
                 order[i] = order[j];
                 order[j] = t;
             }
     int rc = PBS_ERR_TOO_LARGE;
-    for (int i = 0; i < NSHAPES && rc == PBS_ERR_TOO_LARGE; ++i) {
-        const int c = order[i];
+    for (int i = 0; i < NCAND && rc == PBS_ERR_TOO_LARGE; ++i) {
+        if (cost[order[i]] >= 1e300) break;
+        const int wi = order[i] / NSHAPES, c = order[i] % NSHAPES;
+        DdsArgs gw = g;
+        gw.plan = reinterpret_cast<const int*>(reinterpret_cast<const unsigned char*>(g.plan) + narrow_plan_offset(g.N, g.K, wi));
+        gw.n_groups = (int)narrow_groups(g.N, wi);
         if constexpr (sizeof(T) == 4) {
-            rc = c == 0 ? launch_dds<T, TRANS, 2, 1, 3, 8, 0>(g, stream)
-                 : c == 1 ? launch_dds<T, TRANS, 1, 1, 3, 8, 0>(g, stream)
-                 : c == 2 ? launch_dds<T, TRANS, 1, 1, 3, 8, 0, 2>(g, stream)
-                          : launch_dds<T, TRANS, 1, 1, 3, 8, 0, 8, 8>(g, stream);
+            rc = c == 0 ? launch_dds<T, TRANS, 2, 1, 3, 8, 0>(gw, stream)
+                 : c == 1 ? launch_dds<T, TRANS, 1, 1, 3, 8, 0>(gw, stream)
+                 : c == 2 ? launch_dds<T, TRANS, 1, 1, 3, 8, 0, 2>(gw, stream)
+                          : launch_dds<T, TRANS, 1, 1, 3, 8, 0, 8, 8>(gw, stream);
         } else {
-            rc = c == 0 ? launch_dds<T, TRANS, 2, 2, 3, 16, 4>(g, stream)
-                 : c == 1 ? launch_dds<T, TRANS, 1, 2, 3, 16, 4>(g, stream)
-                          : launch_dds<T, TRANS, 1, 2, 3, 16, 4, 2>(g, stream);
+            rc = c == 0 ? launch_dds<T, TRANS, 2, 2, 3, 16, 4>(gw, stream)
+                 : c == 1 ? launch_dds<T, TRANS, 1, 2, 3, 16, 4>(gw, stream)
+                          : launch_dds<T, TRANS, 1, 2, 3, 16, 4, 2>(gw, stream);
         }
     }
     return rc;
 }
 
 // ---- sparse-output product ----
-// fp32: 8 x 8 rectangles, 16-token chunks staged through registers; bf16: 16 x 16 rectangles,
-// 32-token chunks by DMA.
+// fp32: rectangles of 8 x 8, 16 x 8 or 8 x 16 block positions, 16-token chunks staged through registers;
+// bf16: 16 x 16 rectangles, 32-token chunks by DMA.
 struct SddShapeF32 {
-    static constexpr int SR = 8, SC = 8, QW = 8, NW = 8, TC = 16;
+    int SR, SC, QW;
 };
+constexpr int SDD_F32_NSHAPES = 3;
+constexpr SddShapeF32 SDD_F32_SHAPES[SDD_F32_NSHAPES] = {{8, 8, 8}, {16, 8, 10}, {8, 16, 10}};
+constexpr int SDD_F32_NW = 8, SDD_F32_TC = 16;
 struct SddShapeBf16 {
     static constexpr int SR = 16, SC = 16, QW = 10, TC = 32, NS = 2, NW = 8;
 };
 
 struct SddPlan {
     int tiles_r, tiles_c, nsplit, tokens_per_split;
+    int shape;   // fp32: index into SDD_F32_SHAPES
 };
 
 static SddPlan plan_sdd(long long M, int N, int K, int SR, int SC, int TC) {
     SddPlan p;
+    p.shape = 0;
     p.tiles_r = (N / 32 + SR - 1) / SR;
     p.tiles_c = (K / 32 + SC - 1) / SC;
     const long long tiles = (long long)p.tiles_r * p.tiles_c;
@@ -198,14 +249,59 @@ static SddPlan plan_sdd(long long M, int N, int K, int SR, int SC, int TC) {
     p.tokens_per_split = (int)(chunks_per * TC);
     return p;
 }
-static SddPlan plan_sdd_for(int dtype, long long M, int N, int K) {
-    if (dtype == PBS_DTYPE_F32) return plan_sdd(M, N, K, SddShapeF32::SR, SddShapeF32::SC, SddShapeF32::TC);
+// fp32: which rectangle shape.  A workgroup's time per chunk is set by its busiest wave, i.e. by
+// ceil(blocks in the rectangle / 8), and the launch ends with its fullest rectangle; larger rectangles lose
+// less to that rounding (33 blocks on 8 waves cost 5 rounds for 4.1 rounds of work, 66 cost 9 for 8.25)
+// but fit fewer shapes without a ragged last row or column of rectangles, whose workgroups get a full share of
+// the token range for a fraction of the blocks.  The estimate: chunks per workgroup x rounds per chunk for
+// the fullest rectangle expected under a uniform pattern of the given density.
+static SddPlan plan_sdd_f32(long long M, int N, int K, long long nnz) {
+    SddPlan best = plan_sdd(M, N, K, SDD_F32_SHAPES[0].SR, SDD_F32_SHAPES[0].SC, SDD_F32_TC);
+    double best_cost = 0.0;
+    const double positions = (double)(N / 32) * (double)(K / 32);
+    const double d = positions > 0 ? (double)nnz / positions : 0.0;
+    for (int i = 0; i < SDD_F32_NSHAPES; ++i) {
+        const SddShapeF32 sh = SDD_F32_SHAPES[i];
+        SddPlan p = plan_sdd(M, N, K, sh.SR, sh.SC, SDD_F32_TC);
+        p.shape = i;
+        const int sr = N / 32 < sh.SR ? N / 32 : sh.SR, sc = K / 32 < sh.SC ? K / 32 : sh.SC;
+        const double mean = sr * sc * d;
+        const double full = (double)((N / 32) / sh.SR > 0 ? (N / 32) / sh.SR : 1) * ((K / 32) / sh.SC > 0 ? (K / 32) / sh.SC : 1);
+        const double spread = std::sqrt(mean * (1.0 - d)) * std::sqrt(2.0 * std::log(full < 2.0 ? 2.0 : full));
+        double fullest = mean + spread;
+        if (fullest > sr * sc) fullest = sr * sc;
+        double rounds = std::ceil(fullest / SDD_F32_NW);
+        if (rounds < 1.0) rounds = 1.0;
+        if (fullest > sh.QW * SDD_F32_NW) rounds *= 2.0;   // a second pass over the tokens
+        const double chunks_per = (double)p.tokens_per_split / SDD_F32_TC;
+        const double cost = chunks_per * (rounds + 0.5);   // + the chunk's staging and barriers
+        if (i == 0 || cost < best_cost * 0.97) {
+            best = p;
+            best_cost = cost;
+        }
+    }
+    return best;
+}
+static SddPlan plan_sdd_for(int dtype, long long M, int N, int K, long long nnz) {
+    if (dtype == PBS_DTYPE_F32) return plan_sdd_f32(M, N, K, nnz);
     return plan_sdd(M, N, K, SddShapeBf16::SR, SddShapeBf16::SC, SddShapeBf16::TC);
+}
+
+template <int SHAPE>
+static int launch_sdd_f32(const SddArgs& a, long long wgs, hipStream_t stream) {
+    constexpr SddShapeF32 S = SDD_F32_SHAPES[SHAPE];
+    using C = SddCfg<float, S.SR, S.SC, S.QW, SDD_F32_NW>;
+    static_assert(C::TC == SDD_F32_TC, "plan and kernel must agree on the chunk size");
+    static std::atomic<uint64_t> done{0};
+    auto kernel = sdd_kernel<float, S.SR, S.SC, S.QW, SDD_F32_NW>;
+    if (int rc = raise_lds_limit(kernel, C::LDS_BYTES, done)) return rc;
+    hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)wgs)), dim3(C::NT), C::LDS_BYTES, stream, a);
+    return (int)hipGetLastError();
 }
 
 template <typename T>
 static int launch_sdd(SddArgs a, int dtype, void* workspace, size_t workspace_bytes, hipStream_t stream) {
-    const SddPlan p = plan_sdd_for(dtype, a.M, a.N, a.K);
+    const SddPlan p = plan_sdd_for(dtype, a.M, a.N, a.K, a.nnz);
     a.tiles_r = p.tiles_r;
     a.tiles_c = p.tiles_c;
     a.nsplit = p.nsplit;
@@ -220,13 +316,10 @@ static int launch_sdd(SddArgs a, int dtype, void* workspace, size_t workspace_by
     const long long wgs = (long long)p.tiles_r * p.tiles_c * p.nsplit;
     if (wgs > (1ll << 30)) return PBS_ERR_TOO_LARGE;
     if constexpr (sizeof(T) == 4) {
-        using S = SddShapeF32;
-        using C = SddCfg<T, S::SR, S::SC, S::QW, S::NW>;
-        static_assert(C::TC == S::TC, "plan and kernel must agree on the chunk size");
-        static std::atomic<uint64_t> done{0};
-        auto kernel = sdd_kernel<T, S::SR, S::SC, S::QW, S::NW>;
-        if (int rc = raise_lds_limit(kernel, C::LDS_BYTES, done)) return rc;
-        hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)wgs)), dim3(C::NT), C::LDS_BYTES, stream, a);
+        const int rc = p.shape == 0 ? launch_sdd_f32<0>(a, wgs, stream)
+                       : p.shape == 1 ? launch_sdd_f32<1>(a, wgs, stream)
+                                      : launch_sdd_f32<2>(a, wgs, stream);
+        if (rc) return rc;
     } else {
         using S = SddShapeBf16;
         using C = SddBf16Cfg<S::QW, S::TC, S::NS, S::NW>;
@@ -314,7 +407,7 @@ int pbs_build_indices(const uint8_t* mask, const int64_t* block_ptr, int X, int 
 
 size_t pbs_blocksparse_matmul_plan_bytes(int n, int k) {
     if (n <= 0 || k <= 0 || (n % 32) || (k % 32)) return 0;
-    return narrow_plan_bytes(n, k) + wide_plan_bytes(n, k) + slot_table_bytes(n);
+    return all_plan_bytes(n, k);
 }
 
 int pbs_blocksparse_matmul_plan(const int32_t* ptr, const int32_t* indices, int n, int k, int nnz, void* plan,
@@ -323,13 +416,17 @@ int pbs_blocksparse_matmul_plan(const int32_t* ptr, const int32_t* indices, int 
     if ((long long)nnz > (long long)(n / 32) * (k / 32) || k > (1 << 24)) return PBS_ERR_TOO_LARGE;
     if (!ptr || !plan || (nnz > 0 && !indices)) return PBS_ERR_NULL_POINTER;
     if (!aligned16(plan) || plan_bytes < pbs_blocksparse_matmul_plan_bytes(n, k)) return PBS_ERR_WORKSPACE;
-    const int groups = (n / 32 + DDS_NB - 1) / DDS_NB;
-    int* slots = reinterpret_cast<int*>(static_cast<unsigned char*>(plan) + narrow_plan_bytes(n, k) + wide_plan_bytes(n, k));
-    hipLaunchKernelGGL(dds_slots_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(stream), ptr, n / 32, groups, slots);
-    if (int rc = (int)hipGetLastError()) return rc;
-    hipLaunchKernelGGL(dds_plan_kernel, dim3(groups), dim3(256), 0, static_cast<hipStream_t>(stream), ptr, indices, slots,
-                       n / 32, k / 32, nnz, static_cast<int*>(plan), (int)dds_plan_group_ints(k / 32));
-    if (int rc = (int)hipGetLastError()) return rc;
+    for (int wi = 0; wi < DDS_NWIDTHS; ++wi) {
+        const int groups = (int)narrow_groups(n, wi);
+        int* slots = reinterpret_cast<int*>(static_cast<unsigned char*>(plan) + slot_table_offset(n, k, wi));
+        int* narrow = reinterpret_cast<int*>(static_cast<unsigned char*>(plan) + narrow_plan_offset(n, k, wi));
+        hipLaunchKernelGGL(dds_slots_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(stream), ptr, n / 32, groups,
+                           DDS_WIDTHS[wi], slots);
+        if (int rc = (int)hipGetLastError()) return rc;
+        hipLaunchKernelGGL(dds_plan_kernel, dim3(groups), dim3(256), 0, static_cast<hipStream_t>(stream), ptr, indices,
+                           slots, n / 32, k / 32, nnz, narrow, (int)dds_plan_group_ints(k / 32));
+        if (int rc = (int)hipGetLastError()) return rc;
+    }
     if (wide_plan_bytes(n, k)) {
         const int groups16 = (n / 32 + D16_NB - 1) / D16_NB;
         int* wide = reinterpret_cast<int*>(static_cast<unsigned char*>(plan) + narrow_plan_bytes(n, k));
@@ -374,7 +471,7 @@ size_t pbs_blocksparse_matmul_back_workspace_bytes(int64_t tokens, int out_featu
     if (tokens <= 0 || out_features <= 0 || in_features <= 0 || nnz <= 0) return 0;
     if ((out_features % 32) || (in_features % 32)) return 0;
     if (dtype != PBS_DTYPE_F32 && dtype != PBS_DTYPE_BF16) return 0;
-    const SddPlan p = plan_sdd_for(dtype, tokens, out_features, in_features);
+    const SddPlan p = plan_sdd_for(dtype, tokens, out_features, in_features, nnz);
     if (p.nsplit <= 1) return 0;
     return (size_t)nnz * 1024 * sizeof(float) * p.nsplit;
 }

@@ -67,12 +67,14 @@ def test_plan_argument_checks(lib):
     p = ctypes.c_void_p(0x1000)
     null = ctypes.c_void_p(0)
     nbytes = lib.pbs_blocksparse_matmul_plan_bytes(4096, 4096)
-    narrow = 16 * (128 + 2) * 16 * 4           # 16 groups of 8 block columns, 64-byte records per k-block
+    # narrow plans: groups of 8, 7, 6 and 5 block columns (128 columns -> 16, 19, 22, 26 groups), 64-byte
+    # records per k-block, each with the table of the block column in every one of a group's 8 places
+    narrow = sum(g * (128 + 2) * 16 * 4 for g in (16, 19, 22, 26))
+    slots = sum((g * 8 * 4 + 63) // 64 * 64 for g in (16, 19, 22, 26))   # each table padded to 64 bytes
     wide = 8 * (64 + 2) * 64 * 4 + 256 * 4     # 8 groups of 16, 256-byte records per k-pair, progress table
-    slots = 16 * 8 * 4                         # block column of every place of every group
     assert nbytes == narrow + wide + slots
     # contraction sizes that are not a multiple of 64 have no k-pair plan
-    assert lib.pbs_blocksparse_matmul_plan_bytes(64, 96) == 1 * (3 + 2) * 16 * 4 + 64
+    assert lib.pbs_blocksparse_matmul_plan_bytes(64, 96) == 4 * (1 * (3 + 2) * 16 * 4 + 64)
     assert lib.pbs_blocksparse_matmul_plan_bytes(100, 64) == 0
     f = lib.pbs_blocksparse_matmul_plan
     assert f(p, p, 64, 100, 1, p, 1 << 20, null) == ERR_SHAPE

@@ -252,3 +252,25 @@ def test_long_contraction(cuda, dtype):
         print(f"long contraction {in_f}->{out_f} {dtype}", flush=True)
         m = _matrix(out_f, in_f, None, n_blocks, dtype, cuda, seed=17)
         _check_all(m, (tokens,), dtype, cuda, 17, f"{in_f}->{out_f}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("cols,tokens", [(24, 4096), (24, 16384), (40, 4096), (50, 4096), (13, 16384), (5, 2048)])
+def test_column_groups_of_fewer_than_eight(cuda, dtype, cols, tokens):
+    """Results with few block columns against many tokens: the library regroups the block columns 7, 6 or 5 to
+    a tile (24 columns in 4 groups of 6, 40 in 8 groups of 5, 50 in 8 groups of 7 minus a ragged last one) when
+    that gives every CU a tile.  Values, bias and ragged last groups must not notice which grouping ran;
+    both directions, so the regrouped side is once the output features and once the input features."""
+    wide, narrow = cols * 32, 8 * 32
+    for out_f, in_f in ((wide, narrow), (narrow, wide)):
+        print(f"column groups {in_f}->{out_f} tokens {tokens} {dtype}", flush=True)
+        m = _matrix(out_f, in_f, None, max(1, (out_f // 32) * (in_f // 32) // 2), dtype, cuda, seed=cols)
+        _check_all(m, (tokens,), dtype, cuda, cols + 1, f"{in_f}->{out_f}@{tokens}")
+    g = torch.Generator().manual_seed(cols)
+    x = torch.randn((tokens, narrow), generator=g).to(dtype)
+    bias = torch.randn((wide,), generator=g).to(dtype)
+    m = _matrix(wide, narrow, None, cols * 4, dtype, cuda, seed=cols + 2)
+    coo = m.build_coo_block_index().cpu().numpy()
+    w_dense = O.to_dense(to64(m.data), coo, (wide, narrow))
+    yb = m.reverse_matmul(x.to(cuda), True, bias=bias.to(cuda))
+    assert_close(yb, to64(x) @ w_dense.T + to64(bias)[None, :], dtype, "fwd + bias")
