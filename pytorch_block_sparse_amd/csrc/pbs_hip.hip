@@ -13,6 +13,7 @@
 #include "pbs_index.h"
 #include "pbs_sdd.h"
 #include "pbs_sdd_bf16.h"
+#include "pbs_sdd_seg.h"
 
 namespace pbs {
 
@@ -212,13 +213,14 @@ static int dispatch_dds(const DdsArgs& g, hipStream_t stream) {
 }
 
 // ---- sparse-output product ----
-// fp32: rectangles of 8 x 8, 16 x 8 or 8 x 16 block positions, 16-token chunks staged through registers;
+// fp32: equal shares of the blocks of a band of 16 block rows, 16-token chunks by DMA (pbs_sdd_seg.h); rectangles
+// of 8 x 8 block positions staged through registers (pbs_sdd.h) where that kernel does not apply.
 // bf16: 16 x 16 rectangles, 32-token chunks by DMA.
 struct SddShapeF32 {
     int SR, SC, QW;
 };
-constexpr int SDD_F32_NSHAPES = 3;
-constexpr SddShapeF32 SDD_F32_SHAPES[SDD_F32_NSHAPES] = {{8, 8, 8}, {16, 8, 10}, {8, 16, 10}};
+constexpr int SDD_F32_NSHAPES = 1;
+constexpr SddShapeF32 SDD_F32_SHAPES[SDD_F32_NSHAPES] = {{8, 8, 8}};
 constexpr int SDD_F32_NW = 8, SDD_F32_TC = 16;
 struct SddShapeBf16 {
     static constexpr int SR = 16, SC = 16, QW = 10, TC = 32, NS = 2, NW = 8;
@@ -226,12 +228,18 @@ struct SddShapeBf16 {
 
 struct SddPlan {
     int tiles_r, tiles_c, nsplit, tokens_per_split;
-    int shape;   // fp32: index into SDD_F32_SHAPES
+    int shape;   // fp32: index into SDD_F32_SHAPES, or SDD_F32_SEGMENTS
+    int segs;    // segment kernel: shares per row band
 };
+constexpr int SDD_F32_SEGMENTS = SDD_F32_NSHAPES;
+constexpr int SEG_SR = 16, SEG_QW = 9;
+constexpr int SEG_NSC = 2;
+constexpr int SEG_SC[SEG_NSC] = {16, 20};   // X panel widths of the two builds of the segment kernel
 
 static SddPlan plan_sdd(long long M, int N, int K, int SR, int SC, int TC) {
     SddPlan p;
     p.shape = 0;
+    p.segs = 0;
     p.tiles_r = (N / 32 + SR - 1) / SR;
     p.tiles_c = (K / 32 + SC - 1) / SC;
     const long long tiles = (long long)p.tiles_r * p.tiles_c;
@@ -249,21 +257,18 @@ static SddPlan plan_sdd(long long M, int N, int K, int SR, int SC, int TC) {
     p.tokens_per_split = (int)(chunks_per * TC);
     return p;
 }
-// fp32: which rectangle shape.  A workgroup's time per chunk is set by its busiest wave, i.e. by
-// ceil(blocks in the rectangle / 8), and the launch ends with its fullest rectangle; larger rectangles lose
-// less to that rounding (33 blocks on 8 waves cost 5 rounds for 4.1 rounds of work, 66 cost 9 for 8.25)
-// but fit fewer shapes without a ragged last row or column of rectangles, whose workgroups get a full share of
-// the token range for a fraction of the blocks.  The estimate: chunks per workgroup x rounds per chunk for
-// the fullest rectangle expected under a uniform pattern of the given density.
+// fp32: which kernel, and how the work is cut.  A workgroup's time per chunk of tokens is set by its busiest
+// wave, i.e. by rounds = ceil(blocks of the workgroup / 8), and the launch ends with its slowest workgroup.  The
+// estimate for either kernel is chunks per workgroup x (rounds + a half for the chunk's staging and barriers).
+// Rectangles: the fullest of the rectangles expected under a uniform pattern of the given density (33 blocks
+// on 8 waves cost 5 rounds for 4.1 rounds of work).
 static SddPlan plan_sdd_f32(long long M, int N, int K, long long nnz) {
-    SddPlan best = plan_sdd(M, N, K, SDD_F32_SHAPES[0].SR, SDD_F32_SHAPES[0].SC, SDD_F32_TC);
-    double best_cost = 0.0;
+    const SddShapeF32 sh = SDD_F32_SHAPES[0];
+    SddPlan best = plan_sdd(M, N, K, sh.SR, sh.SC, SDD_F32_TC);
     const double positions = (double)(N / 32) * (double)(K / 32);
     const double d = positions > 0 ? (double)nnz / positions : 0.0;
-    for (int i = 0; i < SDD_F32_NSHAPES; ++i) {
-        const SddShapeF32 sh = SDD_F32_SHAPES[i];
-        SddPlan p = plan_sdd(M, N, K, sh.SR, sh.SC, SDD_F32_TC);
-        p.shape = i;
+    double best_cost;
+    {
         const int sr = N / 32 < sh.SR ? N / 32 : sh.SR, sc = K / 32 < sh.SC ? K / 32 : sh.SC;
         const double mean = sr * sc * d;
         const double full = (double)((N / 32) / sh.SR > 0 ? (N / 32) / sh.SR : 1) * ((K / 32) / sh.SC > 0 ? (K / 32) / sh.SC : 1);
@@ -273,11 +278,47 @@ static SddPlan plan_sdd_f32(long long M, int N, int K, long long nnz) {
         double rounds = std::ceil(fullest / SDD_F32_NW);
         if (rounds < 1.0) rounds = 1.0;
         if (fullest > sh.QW * SDD_F32_NW) rounds *= 2.0;   // a second pass over the tokens
-        const double chunks_per = (double)p.tokens_per_split / SDD_F32_TC;
-        const double cost = chunks_per * (rounds + 0.5);   // + the chunk's staging and barriers
-        if (i == 0 || cost < best_cost * 0.97) {
-            best = p;
-            best_cost = cost;
+        best_cost = (double)best.tokens_per_split / SDD_F32_TC * (rounds + 0.5);
+    }
+    // Equal shares of each row band's blocks (pbs_sdd_seg.h): every workgroup does `rounds` products per chunk.
+    // A share of 8 x rounds blocks spans about that many / (rows x density) block columns, which must fit the
+    // kernel's X panel; bands differ a little in their block counts, so the shares are sized for a band two
+    // standard deviations above the mean.  Of the feasible rounds the one with the smallest chunks x rounds wins.
+    const int nblk_r = N / 32, ncols = K / 32;
+    for (int v = 0; v < SEG_NSC; ++v) {
+        // the histogram of a band's block columns borrows the stage buffers
+        const int max_cols = 2 * 16 * (SEG_SR + SEG_SC[v]) * 128 / 4 - 64;
+        if (ncols > max_cols || nnz <= 0 || d <= 0.0) continue;
+        const int bands = (nblk_r + SEG_SR - 1) / SEG_SR;
+        const int rows_per_band = (nblk_r + bands - 1) / bands;
+        const double n_band = (double)nnz * rows_per_band / nblk_r;
+        const double heavy = n_band + (bands > 1 ? 2.0 * std::sqrt(n_band * (1.0 - d)) : 0.0);
+        const long long chunks = (M + SDD_F32_TC - 1) / SDD_F32_TC;
+        for (int q = 1; q <= SEG_QW; ++q) {
+            const double share = 8.0 * q;
+            if (share / (rows_per_band * d) + 2.0 > SEG_SC[v]) break;   // wider than the X panel
+            long long segs = (long long)std::ceil(heavy / share);
+            if (segs < 1) segs = 1;
+            const long long wgs1 = (long long)bands * segs;
+            long long want = 256 / wgs1, cap = chunks / 8;
+            if (cap < 1) cap = 1;
+            if (want > cap) want = cap;
+            if (want < 1) want = 1;
+            const long long chunks_per = (chunks + want - 1) / want;
+            const long long nsplit = (chunks + chunks_per - 1) / chunks_per;
+            const double waves_of_wgs = std::ceil((double)(wgs1 * nsplit) / 256.0);
+            const double rounds = std::ceil(n_band / segs / 8.0);
+            // the wider panel costs a few per cent (more bytes staged per chunk)
+            const double cost = (double)chunks_per * (rounds + 0.5) * waves_of_wgs * (1.0 + 0.04 * v);
+            if (cost < best_cost) {
+                best_cost = cost;
+                best.shape = SDD_F32_SEGMENTS + v;
+                best.tiles_r = bands;
+                best.tiles_c = 1;
+                best.segs = (int)segs;
+                best.nsplit = (int)nsplit;
+                best.tokens_per_split = (int)(chunks_per * SDD_F32_TC);
+            }
         }
     }
     return best;
@@ -299,6 +340,18 @@ static int launch_sdd_f32(const SddArgs& a, long long wgs, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
+template <int V>
+static int launch_sdd_seg(const SddArgs& a, long long wgs, hipStream_t stream) {
+    using C = SddSegCfg<SEG_SR, SEG_SC[V], SEG_QW, SDD_F32_NW>;
+    static_assert(C::MAX_COLS == 2 * 16 * (SEG_SR + SEG_SC[V]) * 128 / 4 - 64, "the plan's column limit is the kernel's");
+    static_assert(C::TC == SDD_F32_TC, "plan and kernel must agree on the chunk size");
+    static std::atomic<uint64_t> done{0};
+    auto kernel = sdd_seg_kernel<SEG_SR, SEG_SC[V], SEG_QW, SDD_F32_NW>;
+    if (int rc = raise_lds_limit(kernel, C::LDS_BYTES, done)) return rc;
+    hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)wgs)), dim3(C::NT), C::LDS_BYTES, stream, a);
+    return (int)hipGetLastError();
+}
+
 template <typename T>
 static int launch_sdd(SddArgs a, int dtype, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     const SddPlan p = plan_sdd_for(dtype, a.M, a.N, a.K, a.nnz);
@@ -306,6 +359,7 @@ static int launch_sdd(SddArgs a, int dtype, void* workspace, size_t workspace_by
     a.tiles_c = p.tiles_c;
     a.nsplit = p.nsplit;
     a.tokens_per_split = p.tokens_per_split;
+    a.segs = p.segs;
     a.partial = nullptr;
     const size_t n = (size_t)a.nnz * 1024;
     if (p.nsplit > 1) {
@@ -313,12 +367,12 @@ static int launch_sdd(SddArgs a, int dtype, void* workspace, size_t workspace_by
         if (!workspace || workspace_bytes < need || !aligned16(workspace)) return PBS_ERR_WORKSPACE;
         a.partial = static_cast<float*>(workspace);
     }
-    const long long wgs = (long long)p.tiles_r * p.tiles_c * p.nsplit;
+    const long long wgs = (long long)p.tiles_r * (p.segs > 0 ? p.segs : p.tiles_c) * p.nsplit;
     if (wgs > (1ll << 30)) return PBS_ERR_TOO_LARGE;
     if constexpr (sizeof(T) == 4) {
-        const int rc = p.shape == 0 ? launch_sdd_f32<0>(a, wgs, stream)
-                       : p.shape == 1 ? launch_sdd_f32<1>(a, wgs, stream)
-                                      : launch_sdd_f32<2>(a, wgs, stream);
+        const int rc = p.shape == SDD_F32_SEGMENTS ? launch_sdd_seg<0>(a, wgs, stream)
+                       : p.shape == SDD_F32_SEGMENTS + 1 ? launch_sdd_seg<1>(a, wgs, stream)
+                                                         : launch_sdd_f32<0>(a, wgs, stream);
         if (rc) return rc;
     } else {
         using S = SddShapeBf16;
@@ -507,7 +561,7 @@ int pbs_blocksparse_matmul_back(const void* dense_a, const void* dense_b, const 
     a.N = out_features;
     a.K = in_features;
     a.nnz = nnz;
-    a.tiles_r = a.tiles_c = a.nsplit = a.tokens_per_split = 0;
+    a.tiles_r = a.tiles_c = a.nsplit = a.tokens_per_split = a.segs = 0;
     if (dtype == PBS_DTYPE_F32) return launch_sdd<float>(a, dtype, workspace, workspace_bytes, s);
     return launch_sdd<bf16_t>(a, dtype, workspace, workspace_bytes, s);
 }

@@ -23,6 +23,7 @@ struct SddArgs {
     int M, N, K, nnz;
     int tiles_r, tiles_c, nsplit;
     int tokens_per_split;    // multiple of TC
+    int segs;                // segment kernel: equal shares of a row band's blocks (tiles_c is unused there)
 };
 
 // Which block rows of W form row band `band` of rectangles (SR places; -1 = no row).  Normally they are
@@ -35,7 +36,8 @@ struct SddArgs {
 constexpr int SDD_BALANCE_MAX_ROWS = 1024;
 static __device__ __forceinline__ bool sdd_band_rows(const int32_t* __restrict__ ptr, int nnz, int nblk_r, int tiles_r, int band,
                                                      int SR, int* s_rowid, int* scratch, int tid, int nthreads,
-                                                     int* s_ptr_copy = nullptr) {
+                                                     int* s_ptr_copy = nullptr, int rows_per_band = 0) {
+    if (rows_per_band <= 0 || rows_per_band > SR) rows_per_band = SR;   // natural order: rows band * rows_per_band ...
     bool skewed = false;
     const bool scanned = nblk_r <= SDD_BALANCE_MAX_ROWS && tiles_r >= 2;
     if (scanned) {
@@ -61,8 +63,8 @@ static __device__ __forceinline__ bool sdd_band_rows(const int32_t* __restrict__
         skewed = (long long)*s_max * nblk_r > 2ll * *s_sum;
     }
     if (tid < SR) {
-        const int r = band * SR + tid;
-        s_rowid[tid] = (!skewed && r < nblk_r) ? r : -1;
+        const int r = band * rows_per_band + tid;
+        s_rowid[tid] = (!skewed && tid < rows_per_band && r < nblk_r) ? r : -1;
     }
     __syncthreads();
     if (skewed) {

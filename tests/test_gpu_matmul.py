@@ -274,3 +274,24 @@ def test_column_groups_of_fewer_than_eight(cuda, dtype, cols, tokens):
     w_dense = O.to_dense(to64(m.data), coo, (wide, narrow))
     yb = m.reverse_matmul(x.to(cuda), True, bias=bias.to(cuda))
     assert_close(yb, to64(x) @ w_dense.T + to64(bias)[None, :], dtype, "fwd + bias")
+
+
+def test_weight_gradient_equal_shares_on_uneven_patterns(cuda):
+    """The fp32 weight-gradient kernel cuts each band of 16 block rows into shares of equal block count and sizes
+    the shares for a uniform pattern.  Patterns that are far from uniform take its slow paths, which must still be
+    exact: (a) a share that spans more block columns than its X panel holds is done in several column windows;
+    (b) a band much denser than the average gives shares with more blocks than a workgroup has accumulators
+    for, done in several passes; (c) a share boundary inside a block column splits that column between two
+    workgroups.  Ragged token counts on top (the last chunk is padded with zeros in LDS)."""
+    dtype = torch.float32
+    # (a) 16 x 256 block positions: 8 full columns, then one block in every other column
+    blocks_a = [(r, c) for c in range(8) for r in range(16)] + [((c * 7) % 16, c) for c in range(8, 256, 2)]
+    # (b) 64 x 32: the first band full, one block per row below it
+    blocks_b = [(r, c) for r in range(16) for c in range(32)] + [(r, (5 * r) % 32) for r in range(16, 64)]
+    # (c) 16 x 6, every position present, 96 blocks: shares cut columns in the middle
+    blocks_c = [(r, c) for r in range(16) for c in range(6)]
+    for name, grid, blocks, tokens in (("windows", (16, 256), blocks_a, 209), ("passes", (64, 32), blocks_b, 333),
+                                       ("split columns", (16, 6), blocks_c, 4099)):
+        print(f"equal shares: {name}", flush=True)
+        m = _matrix(grid[0] * 32, grid[1] * 32, blocks, None, dtype, cuda, seed=len(blocks))
+        _check_all(m, (tokens,), dtype, cuda, 23, name)
