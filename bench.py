@@ -10,7 +10,8 @@ Prints ONE JSON line: effective TFLOP/s (2*M*nnz*1024 per GEMM, 3 GEMMs per step
   dense_hipblaslt  the same three GEMMs dense through torch.matmul (hipBLASLt) at the same shape,
   cpu_baseline   the CPU dense-equivalent path (oracle) timed on the host cores, full size,
   other_configs  the other benchmark configurations (1024->256 forward, the two RoBERTa feed-forward
-                 shapes in fp32, the RoBERTa-base training step), each with its own dense comparison.
+                 shapes in fp32, the 4096 x 4096 layer in fp32, the RoBERTa-base training step), each with its own
+                 dense comparison.
 
 Timing: after a settling phase and `--warmup` untimed steps, exactly `--steps` steps are timed between two
 synchronisations; an event is recorded after every kernel of every timed step.  `ms_per_step` and `value`
@@ -34,7 +35,8 @@ HBM_TBPS = 8.0
 # not reported (null).
 BASELINE_WORKLOAD = "c4_4096x4096_d0.25_bf16"
 BASELINE_METRIC = "effective TFLOP/s fwd+bwd at 4096² d=0.25; % of MFMA peak; vs dense GEMM"   # as in BASELINE.json
-OTHER_LAYER_WORKLOADS = ("c1_1024x256_d0.1_fp32", "c2_768x3072_d0.5_fp32", "c3_3072x768_d0.25_zipf_fp32")
+OTHER_LAYER_WORKLOADS = ("c1_1024x256_d0.1_fp32", "c2_768x3072_d0.5_fp32", "c3_3072x768_d0.25_zipf_fp32",
+                         "c4_4096x4096_d0.25_fp32")   # the last: the headline shape in the reference's own dtype
 ROBERTA_WORKLOAD = "c5_roberta_base_mlm_fp32"
 
 
