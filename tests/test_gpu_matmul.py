@@ -295,3 +295,36 @@ def test_weight_gradient_equal_shares_on_uneven_patterns(cuda):
         print(f"equal shares: {name}", flush=True)
         m = _matrix(grid[0] * 32, grid[1] * 32, blocks, None, dtype, cuda, seed=len(blocks))
         _check_all(m, (tokens,), dtype, cuda, 23, name)
+
+
+def test_benchmark_shape_fp32_4096(cuda):
+    """4096 -> 4096, density 0.25, fp32 (the headline shape in the reference's dtype): oracle-checked on the first
+    3072 tokens (the oracle is three dense fp64 products), and at the full 16384 tokens through the adjoint identity
+    <dY, X W^T> == <dY W, X> == <dW, W> and token additivity of dW, which tie the three kernels together."""
+    w = workloads.WORKLOADS["c4_4096x4096_d0.25_fp32"]
+    blocks, data, x, dy = workloads.make_inputs(w)
+    m = BlockSparseMatrix.zeros((w.out_features, w.in_features), blocks=blocks, device="cpu", dtype=w.dtype)
+    with torch.no_grad():
+        m.data.copy_(data)
+    m = m.to(cuda)
+    coo = m.build_coo_block_index().cpu().numpy()
+    part = 3072
+    y_ref, dx_ref, dw_ref = O.linear_fwd_bwd(to64(x[:part]), to64(dy[:part]), to64(data), coo, tuple(m.shape))
+    xd, dyd = x.to(cuda), dy.to(cuda)
+    assert_close(m.reverse_matmul(xd[:part], True), y_ref, w.dtype, "fwd")
+    assert_close(m.reverse_matmul(dyd[:part], False), dx_ref, w.dtype, "dx")
+    assert_close(m.matmul_with_output_sparse_support(dyd[:part], xd[:part]), dw_ref, w.dtype, "dw")
+    y = m.reverse_matmul(xd, True)
+    dx = m.reverse_matmul(dyd, False)
+    dw = m.matmul_with_output_sparse_support(dyd, xd)
+    a = (dyd.double() * y.double()).sum().item()
+    b = (dx.double() * xd.double()).sum().item()
+    c = (dw.double() * m.data.double()).sum().item()
+    scale = (dyd.double().norm() * y.double().norm()).item()
+    print("adjoint", a, b, c, scale, flush=True)
+    assert abs(a - b) < 1e-5 * scale and abs(a - c) < 1e-5 * scale
+    half = w.tokens // 2
+    ref = (m.matmul_with_output_sparse_support(dyd[:half], xd[:half]).double()
+           + m.matmul_with_output_sparse_support(dyd[half:], xd[half:]).double())
+    assert (dw.double() - ref).abs().max().item() < 1e-4 * ref.abs().max().item()
+    assert torch.equal(m.reverse_matmul(xd[1024:1536], True), y[1024:1536])
