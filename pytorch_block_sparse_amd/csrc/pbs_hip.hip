@@ -157,12 +157,17 @@ static int dispatch_dds(const DdsArgs& g, hipStream_t stream) {
     // shapes: 0 = 256 x 8 (4 token slices x 2 column halves), 1 = 128 x 8, 2 = 128 x 4,
     //         3 = 256 x 8 with 8 token slices (every wave has all 8 columns; fp32 only: 8 accumulators of fp32
     //             fragments fit the registers, and balanced waves are worth more than the larger fragments cost)
+    //         4 = 128 x 4 with one k-block per step (fp32 only).  The fp32 shapes of 128 tokens take two k-blocks
+    //             per step in two ring stages: their steps are short (a k-block is one or two block products per
+    //             wave), so a barrier per k-block costs them a fifth of their time (768 -> 3072 input gradient at
+    //             4096 tokens 0.142 -> 0.116 ms); shape 4 needs half the LDS and is what very long contractions
+    //             fall through to.
     // widths: 8, 7, 6 or 5 of a tile's 8 (4) places hold a block column.  A tile's time falls with the columns it
     //         holds, though not in proportion (its panel traffic and per-step overhead stay); bf16 tiles are
     //         bound by their operand stream rather than by the matrix cores and gain less.
-    constexpr int NSHAPES = sizeof(T) == 4 ? 4 : 3;
+    constexpr int NSHAPES = sizeof(T) == 4 ? 5 : 3;
     constexpr int NCAND = NSHAPES * DDS_NWIDTHS;
-    const double area[4] = {2048.0, 1024.0 * 1.04, 512.0 * 1.10, 2048.0 * 0.8};
+    const double area[5] = {2048.0, 1024.0 * 1.04, 512.0 * 1.10, 2048.0 * 0.8, 512.0 * 1.35};
     const double fixed = sizeof(T) == 4 ? 0.15 : 0.35;   // share of a tile's time that does not depend on its columns
     double cost[NCAND];
     int order[NCAND];
@@ -171,11 +176,12 @@ static int dispatch_dds(const DdsArgs& g, hipStream_t stream) {
         // of the widths that give the same number of groups only the narrowest (most even) is tried
         const bool useful = wi == 0 || (groups > (long long)narrow_groups(g.N, 0) &&
                                         (wi == DDS_NWIDTHS - 1 || groups != (long long)narrow_groups(g.N, wi + 1)));
-        const long long tiles[4] = {
+        const long long tiles[5] = {
             (long long)((g.M + 255) / 256) * groups,
             (long long)((g.M + 127) / 128) * groups,
             (long long)((g.M + 127) / 128) * groups * 2,
             (long long)((g.M + 255) / 256) * groups,
+            (long long)((g.M + 127) / 128) * groups * 2,
         };
         for (int c = 0; c < NSHAPES; ++c) {
             const int i = wi * NSHAPES + c;
@@ -200,9 +206,10 @@ static int dispatch_dds(const DdsArgs& g, hipStream_t stream) {
         gw.n_groups = (int)narrow_groups(g.N, wi);
         if constexpr (sizeof(T) == 4) {
             rc = c == 0 ? launch_dds<T, TRANS, 2, 1, 3, 8, 0>(gw, stream)
-                 : c == 1 ? launch_dds<T, TRANS, 1, 1, 3, 8, 0>(gw, stream)
-                 : c == 2 ? launch_dds<T, TRANS, 1, 1, 3, 8, 0, 2>(gw, stream)
-                          : launch_dds<T, TRANS, 1, 1, 3, 8, 0, 8, 8>(gw, stream);
+                 : c == 1 ? launch_dds<T, TRANS, 1, 2, 2, 16, 0>(gw, stream)
+                 : c == 2 ? launch_dds<T, TRANS, 1, 2, 2, 16, 0, 2>(gw, stream)
+                 : c == 3 ? launch_dds<T, TRANS, 1, 1, 3, 8, 0, 8, 8>(gw, stream)
+                          : launch_dds<T, TRANS, 1, 1, 3, 8, 0, 2>(gw, stream);
         } else {
             rc = c == 0 ? launch_dds<T, TRANS, 2, 2, 3, 16, 4>(gw, stream)
                  : c == 1 ? launch_dds<T, TRANS, 1, 2, 3, 16, 4>(gw, stream)
