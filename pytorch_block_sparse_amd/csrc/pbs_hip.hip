@@ -157,6 +157,10 @@ static int dispatch_dds(const DdsArgs& g, hipStream_t stream) {
     // shapes: 0 = 256 x 8 (4 token slices x 2 column halves), 1 = 128 x 8, 2 = 128 x 4,
     //         3 = 256 x 8 with 8 token slices (every wave has all 8 columns; fp32 only: 8 accumulators of fp32
     //             fragments fit the registers, and balanced waves are worth more than the larger fragments cost)
+    //         fp32 shapes 1 to 3 have four copy waves beside the eight compute waves (their registers allow three
+    //         waves per SIMD): a compute wave that also issues the DMA spends 900 to 1400 cycles of every step on
+    //         it, at the start of the step when no wave of its SIMD has products in flight (4096 x 4096 forward
+    //         1.37 -> 1.27 ms).  Shape 0 needs 200 registers per lane and keeps copying with its compute waves.
     //         4 = 128 x 4 with one k-block per step (fp32 only).  The fp32 shapes of 128 tokens take two k-blocks
     //             per step in two ring stages: their steps are short (a k-block is one or two block products per
     //             wave), so a barrier per k-block costs them a fifth of their time (768 -> 3072 input gradient at
@@ -206,9 +210,9 @@ static int dispatch_dds(const DdsArgs& g, hipStream_t stream) {
         gw.n_groups = (int)narrow_groups(g.N, wi);
         if constexpr (sizeof(T) == 4) {
             rc = c == 0 ? launch_dds<T, TRANS, 2, 1, 3, 8, 0>(gw, stream)
-                 : c == 1 ? launch_dds<T, TRANS, 1, 2, 2, 16, 0>(gw, stream)
-                 : c == 2 ? launch_dds<T, TRANS, 1, 2, 2, 16, 0, 2>(gw, stream)
-                 : c == 3 ? launch_dds<T, TRANS, 1, 1, 3, 8, 0, 8, 8>(gw, stream)
+                 : c == 1 ? launch_dds<T, TRANS, 1, 2, 2, 16, 4>(gw, stream)
+                 : c == 2 ? launch_dds<T, TRANS, 1, 2, 2, 16, 4, 2>(gw, stream)
+                 : c == 3 ? launch_dds<T, TRANS, 1, 1, 3, 8, 4, 8, 8>(gw, stream)
                           : launch_dds<T, TRANS, 1, 1, 3, 8, 0, 2>(gw, stream);
         } else {
             rc = c == 0 ? launch_dds<T, TRANS, 2, 2, 3, 16, 4>(gw, stream)
