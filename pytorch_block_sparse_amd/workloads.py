@@ -54,6 +54,9 @@ WORKLOADS = {
     "c4_4096x4096_d0.25_bf16": Workload("c4_4096x4096_d0.25_bf16", 4096, 4096, 0.25, 16384, torch.bfloat16),
     # the headline shape in the reference's own dtype
     "c4_4096x4096_d0.25_fp32": Workload("c4_4096x4096_d0.25_fp32", 4096, 4096, 0.25, 16384, torch.float32),
+    # the headline shape at the upper end of the density range the speed-up over dense is asked for
+    "c4_4096x4096_d0.5_bf16": Workload("c4_4096x4096_d0.5_bf16", 4096, 4096, 0.5, 16384, torch.bfloat16),
+    "c4_4096x4096_d0.5_fp32": Workload("c4_4096x4096_d0.5_fp32", 4096, 4096, 0.5, 16384, torch.float32),
     # the three linear layers patched in every encoder layer of the RoBERTa-base training step
     # (attention.output.dense, intermediate.dense, output.dense) at its 32 x 512 tokens
     "c5_attn_out_768x768_d0.5_fp32": Workload("c5_attn_out_768x768_d0.5_fp32", 768, 768, 0.5, 16384, torch.float32),
