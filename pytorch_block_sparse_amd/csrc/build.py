@@ -1,13 +1,24 @@
-"""Compile libpbs_hip.so (the C-ABI HIP library) for gfx950 next to its sources."""
+"""Compile libpbs_hip.so (the C-ABI HIP library) for gfx950 next to its sources.
+
+Also libpbs_hip_check.so: the same library with the wide bf16 kernel's conservative progress protocol
+(-DPBS_DDS16_PUBLISH_AFTER_WAIT).  Only tests/test_gpu_wide_protocol.py loads it, to compare the two bit for bit.
+"""
 import os
 import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(HERE, "libpbs_hip.so")
+CHECK_LIB = os.path.join(HERE, "libpbs_hip_check.so")
 
 
 def build(verbose=True):
+    _compile(LIB, [], verbose)
+    _compile(CHECK_LIB, ["-DPBS_DDS16_PUBLISH_AFTER_WAIT"], verbose)
+    return LIB
+
+
+def _compile(lib, defines, verbose):
     cmd = [
         os.environ.get("HIPCC", "hipcc"),
         "-O3",
@@ -19,8 +30,9 @@ def build(verbose=True):
         "-target-feature",
         "-Xclang",
         "-packed-fp32-ops",
+        *defines,
         "-o",
-        LIB,
+        lib,
         os.path.join(HERE, "pbs_hip.hip"),
     ]
     if verbose:
@@ -32,7 +44,7 @@ def build(verbose=True):
         print(out)
     if res.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + res.stdout)
-    return LIB
+    return lib
 
 
 if __name__ == "__main__":

@@ -334,8 +334,16 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
                 if (t + 1 < nsteps) enter_tile(jn);
             }
             vrec = fetch_rec(sn);   // consumed in the next iteration: the LDS latency is hidden
+#ifdef PBS_DDS16_PUBLISH_AFTER_WAIT
+            // Checking build (libpbs_hip_check.so): the conservative protocol.  The copy wave waits until all its
+            // loads have returned and only then writes the step number itself, so nothing depends on the order in
+            // which one wave's LDS-DMA loads land.  Slower; its results must equal the product build's bit for bit.
+            wait_dma(0);
+            lds_poke(s_landed + dw * 64 + lane, (t + 1) & 255);
+#else
             // behind the operands of step t: the number t + 1 (mod 256) onto this wave's landed words
             dma4(landed_lds, uniform_ptr(reinterpret_cast<const unsigned char*>(g.seq + ((t + 1) & 255))), 0u);
+#endif
             (void)n_t;
         }
         wait_dma(0);
