@@ -1,0 +1,732 @@
+// dense x block-sparse -> dense for bf16, one block column per wave (forward and input gradient).
+//
+// Tile: 128 tokens x 16 block columns, owned by one workgroup of 16 waves (4 per SIMD).  Wave w owns one
+// block column of the tile for all 128 tokens: four 32 x 32 accumulators with fixed register names.
+// Its work is a list of items, one per stored block of its column, sorted by k; which accumulator a
+// product goes to never depends on the pattern, so the loop over items is straight-line code: 8 loads of
+// dense-operand fragments from LDS, 8 matrix instructions.  Four waves per SIMD cover each other's waits.
+//
+// The block columns are ranked by block count and dealt to the waves so that every SIMD of every
+// workgroup gets the same number of blocks (ddsc_cols_kernel): places 0-3 of a group (one per SIMD) hold
+// its heaviest columns, places 12-15 its lightest.  The waves of the light half (places 8-15) have time to
+// spare and do all the copying; the heavy half only multiplies.
+//
+// Operands.
+//   dense operand   A step is a pair of adjacent k-blocks (128-byte rows).  Its 128 x 64 panel goes
+//                   global -> LDS by DMA into a ring of RS steps (16 KB each).  Step t is copied by the four
+//                   waves 8 + 4 (t % 2) .. + 3, 32 rows = 4 DMA instructions each (a single wave cannot
+//                   issue DMA fast enough).
+//   packed blocks   never pass through LDS.  A block is multiplied by exactly one wave per token tile, so
+//                   the wave loads its two 16-byte fragments per lane straight from global memory into
+//                   registers, L items ahead.  That needs the block stored with k along its rows
+//                   ([n][k]); the stored layout is that for the input gradient, the forward product is
+//                   given a copy of the data with every block transposed (transpose_blocks_kernel).
+//   The LDS so freed makes the panel ring 8 or 9 steps deep, which covers the round trip of a DMA under load.
+//
+// The product is computed transposed, acc[n][token] (block fragment as first operand): a lane then holds
+// 4 consecutive result columns of one token per accumulator register quad; the two lane halves exchange
+// quads (v_permlane32_swap) so that every lane stores 16 contiguous bytes of a result row, straight from
+// the registers.
+//
+// Progress words in LDS (one writer each, only growing; no barriers after the prologue):
+//   landed[c]   steps copied by copier c (wave 8 + c) whose rows have arrived, as (last step + 1) mod 256: behind
+//               its rows of step t the wave issues one single-lane 4-byte DMA that copies the number from a
+//               table in global memory onto the word; a wave's loads complete in order;
+//   done[w]     the global step wave w still needs: it has finished reading every earlier step.
+// Step t may overwrite ring slot t % RS once min done[] > t - RS.  Every step up to min landed[] - 2 has
+// arrived whatever its copiers; a wave remembers that bound and reads the words again only when its next
+// item lies beyond it.  A copier reads them for every item (it also needs min done[]), behind the item's
+// fragment reads, and reduces them after its matrix instructions, so the round trip is off the item's path.
+// Every wait polls with s_sleep and is bounded; a wait that runs into its bound (a broken protocol, not
+// a slow machine) makes the results NaN instead of passing silently.
+//
+// The block loads are ordinary loads: the compiler waits for them where their registers are first used.  It does
+// not see the DMA instructions (inline assembly), so in a copier such a wait covers as many older loads as DMA
+// instructions were issued since the block was requested; the DMA is therefore issued right before that
+// wait, where it is the youngest.  The heavy half issues no DMA and waits exactly.
+//
+// Persistent workgroups: a workgroup keeps one group of 16 block columns and walks several token
+// tiles; steps are numbered across tiles, so the first loads of a tile overlap the previous tile's stores.
+//
+// Plan per group of 16 block columns (ddsc_plan_kernel), ints:
+//   [0] ns = k-pairs any column touches   [1 + c] items of column c   [17] 1 if the lists are usable
+//   [32 + c] block column of the result in place c (or -1)
+//   [64 + s]                  k-pair index of step s
+//   [64 + KP + c * KB + i]    item i of column c: step | (k & 1) << 9 | block << 10   (KP = K / 64, KB = K / 32)
+#pragma once
+#include <type_traits>
+
+#include "pbs_common.h"
+
+namespace pbs {
+
+constexpr int DC_NB = 16;               // block columns per tile = waves per workgroup
+constexpr int DC_NC = 8;                // copiers: the waves DC_NB - DC_NC .. DC_NB - 1
+constexpr int DC_BM = 128;              // tokens per tile
+constexpr int DC_HDR = 64;
+constexpr int DC_H_COL = 32;
+constexpr int DC_MAX_KP = 512;          // k-pairs (K <= 32768): 9 bits of an item
+constexpr int DC_MAX_BLOCKS = 1 << 21;  // block id: 22 bits of an item; byte offsets of blocks stay below 2^32
+constexpr int DC_ITEMS_LDS = 2048;      // items of a group kept in LDS (every pattern up to K = 4096)
+constexpr int DC_SEQ_INTS = 65536;      // the table 0, 1, 2, ...: a workgroup's steps are numbered below this
+#ifndef DC_SLEEP
+#define DC_SLEEP 2
+#endif
+static inline size_t ddsc_plan_group_ints(int KB) { return (size_t)DC_HDR + (KB / 2) + (size_t)DC_NB * KB; }
+
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+// Which block column sits in which place of which group: cols[16 g + c], or -1.  Natural order unless the
+// per-column block counts differ; then the columns are ranked by count and dealt in serpentine order to
+// the SIMD quarters of the groups (place c runs on SIMD c % 4), so that every SIMD of every workgroup gets
+// about the same number of blocks.  One workgroup.
+constexpr int DC_BALANCE_MAX_COLS = 4096;
+__global__ __launch_bounds__(256) void ddsc_cols_kernel(const int32_t* __restrict__ ptr, int nblk_n, int n_groups, int nnz,
+                                                        int* cols) {
+    constexpr int NT = 256;
+    __shared__ int s_cnt[DC_BALANCE_MAX_COLS];
+    const int tid = threadIdx.x;
+    const int total = n_groups * DC_NB;
+    if (nblk_n > DC_BALANCE_MAX_COLS) {
+        for (int i = tid; i < total; i += NT) cols[i] = i < nblk_n ? i : -1;
+        return;
+    }
+    for (int i = tid; i < total; i += NT) cols[i] = -1;
+    for (int c = tid; c < nblk_n; c += NT) s_cnt[c] = clamp_entry(ptr[c + 1], nnz) - clamp_entry(ptr[c], nnz);
+    __syncthreads();
+    const int units = 4 * n_groups;   // SIMD quarters: 4 places each
+    for (int c = tid; c < nblk_n; c += NT) {
+        const int n = s_cnt[c];
+        int rank = 0;
+        for (int o = 0; o < nblk_n; ++o) {
+            const int m = s_cnt[o];
+            rank += (m > n || (m == n && o < c)) ? 1 : 0;
+        }
+        const int turn = rank / units;             // 0..3: which of the quarter's 4 places
+        int u = rank % units;
+        if (turn & 1) u = units - 1 - u;           // serpentine: heavy and light columns pair up
+        // quarter u = (group u / 4, SIMD u % 4); its places are SIMD + 4 * turn
+        cols[(u >> 2) * DC_NB + (u & 3) + 4 * turn] = c;
+    }
+}
+
+// One workgroup per group of 16 block columns.
+__global__ __launch_bounds__(256) void ddsc_plan_kernel(const int32_t* __restrict__ ptr, const int32_t* __restrict__ idx,
+                                                        const int* __restrict__ cols, int nblk_n, int KB, int nnz, int* plan,
+                                                        int group_ints, int* seq) {
+    __shared__ int s_rank[DC_MAX_KP + 1];
+    __shared__ int s_lo[DC_NB], s_hi[DC_NB];
+    __shared__ int s_part[256];
+    const int tid = threadIdx.x;
+    const int KP = KB / 2;
+    int* out = plan + (size_t)blockIdx.x * group_ints;
+    if (tid < DC_NB) {
+        const int c = cols[blockIdx.x * DC_NB + tid];
+        const bool ok = c >= 0 && c < nblk_n;
+        s_lo[tid] = ok ? clamp_entry(ptr[c], nnz) : 0;
+        s_hi[tid] = ok ? clamp_entry(ptr[c + 1], nnz) : 0;
+        out[DC_H_COL + tid] = ok ? c : -1;
+    }
+    for (int i = tid; i <= KP; i += 256) s_rank[i] = 0;
+    __syncthreads();
+    // k-pairs present
+    for (int c = 0; c < DC_NB; ++c)
+        for (int e = s_lo[c] + tid; e < s_hi[c]; e += 256) {
+            const int kb = idx[2 * e], b = idx[2 * e + 1];
+            if (kb >= 0 && kb < KB && b >= 0 && b < nnz) s_rank[kb >> 1] = 1;
+        }
+    __syncthreads();
+    // exclusive prefix sum over the k-pairs (KP <= 512: two per thread, then a scan over 256 partial sums)
+    const int p0 = 2 * tid, p1 = 2 * tid + 1;
+    const int f0 = p0 < KP ? s_rank[p0] : 0, f1 = p1 < KP ? s_rank[p1] : 0;
+    s_part[tid] = f0 + f1;
+    __syncthreads();
+    for (int d = 1; d < 256; d <<= 1) {
+        const int v = tid >= d ? s_part[tid - d] : 0;
+        __syncthreads();
+        s_part[tid] += v;
+        __syncthreads();
+    }
+    const int before = s_part[tid] - (f0 + f1);
+    const int ns = s_part[255];
+    if (p0 < KP) {
+        s_rank[p0] = before;
+        if (f0) out[DC_HDR + before] = p0;
+    }
+    if (p1 < KP) {
+        s_rank[p1] = before + f0;
+        if (f1) out[DC_HDR + before + f0] = p1;
+    }
+    __syncthreads();
+    // items: thread c walks column c's entries (sorted by k; entries that are not are dropped)
+    if (tid < DC_NB) {
+        int* items = out + DC_HDR + KP + (size_t)tid * KB;
+        int n = 0, last = -1;
+        for (int e = s_lo[tid]; e < s_hi[tid]; ++e) {
+            const int kb = idx[2 * e], b = idx[2 * e + 1];
+            if (kb > last && kb < KB && b >= 0 && b < nnz) {
+                items[n++] = s_rank[kb >> 1] | ((kb & 1) << 9) | (b << 10);
+                last = kb;
+            }
+        }
+        out[1 + tid] = n;
+    }
+    if (tid == 0) {
+        out[0] = ns;
+        out[17] = 1;
+    }
+    if (tid >= 18 && tid < DC_H_COL) out[tid] = 0;
+    if (tid >= DC_H_COL + DC_NB && tid < DC_HDR) out[tid] = 0;
+    // the numbers the waves publish their copies with
+    for (int i = blockIdx.x * 256 + tid; i < DC_SEQ_INTS; i += gridDim.x * 256) seq[i] = i;
+}
+
+// data_t block b = data block b transposed (32 x 32 elements of 2 bytes): one wave per block.
+__global__ __launch_bounds__(256) void transpose_blocks_kernel(const uint16_t* __restrict__ data, uint16_t* __restrict__ data_t,
+                                                               int nnz) {
+    __shared__ uint16_t s[4][32][34];
+    const int w = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int b = blockIdx.x * 4 + w;
+    if (b >= nnz) return;
+    const uint16_t* src = data + (size_t)b * 1024;
+    uint16_t* dst = data_t + (size_t)b * 1024;
+    // lane l reads 16 elements: row l / 2, columns 16 (l % 2) .. + 15
+    const int r = lane >> 1, c0 = (lane & 1) * 16;
+    const uint4 v0 = *reinterpret_cast<const uint4*>(src + r * 32 + c0);
+    const uint4 v1 = *reinterpret_cast<const uint4*>(src + r * 32 + c0 + 8);
+    const uint32_t wv[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        s[w][c0 + 2 * i][r] = (uint16_t)(wv[i] & 0xffffu);
+        s[w][c0 + 2 * i + 1][r] = (uint16_t)(wv[i] >> 16);
+    }
+    __builtin_amdgcn_wave_barrier();
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    uint32_t o[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = (uint32_t)s[w][r][c0 + 2 * i] | ((uint32_t)s[w][r][c0 + 2 * i + 1] << 16);
+    *reinterpret_cast<uint4*>(dst + r * 32 + c0) = make_uint4(o[0], o[1], o[2], o[3]);
+    *reinterpret_cast<uint4*>(dst + r * 32 + c0 + 8) = make_uint4(o[4], o[5], o[6], o[7]);
+}
+
+
+
+struct DdscArgs {
+    const void* a;         // [M, K] row-major bf16
+    const void* data;      // [nnz*32, 32] bf16, every block stored [n][k]
+    const int* plan;       // built by ddsc_plan_kernel for this pattern and direction
+    const int* seq;        // the table 0..255 written by ddsc_plan_kernel
+    const void* bias;      // nullptr or [N]
+    void* out;             // [M, N] row-major
+    int M, N, K, nnz;
+    int m_tiles, n_groups, group_ints;
+    int wg_per_group;      // workgroups that share the token tiles of one column group
+#ifdef DC_PROF
+    long long* prof;
+#endif
+};
+
+template <int RS>
+struct DdscCfg {
+    static constexpr int NW = DC_NB, NT = NW * 64, BM = DC_BM;
+    static constexpr int ROWB = 128;                   // one panel row: 64 k values
+    static constexpr int PANEL_BYTES = BM * ROWB;      // 16 KB per step
+    static constexpr int A_RING_BYTES = RS * PANEL_BYTES;
+    static constexpr int ITEMS_OFF = A_RING_BYTES;
+    static constexpr int STEPS_OFF = ITEMS_OFF + DC_ITEMS_LDS * 4;
+    static constexpr int FLAG_OFF = STEPS_OFF + DC_MAX_KP * 4;
+    static constexpr int LDS_BYTES = FLAG_OFF + 256;   // landed[8], done[16], failure word
+    static constexpr int SPIN_LIMIT = 1 << 18;
+    static_assert(RS >= 4 && RS <= 9, "ring depth");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS");
+};
+
+// 4-byte DMA with only lane 0 active: the word at base to the LDS word at lds_base
+static __device__ __forceinline__ void dma4_lane0(unsigned lds_base_uniform, const unsigned char* base_uniform) {
+    uint64_t saved;
+    lds_base_uniform = __builtin_amdgcn_readfirstlane(lds_base_uniform);
+    asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, 1\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %2, %3\n\ts_mov_b64 exec, %0\n\t"
+                 : "=&s"(saved)
+                 : "s"(lds_base_uniform), "v"(0u), "s"(base_uniform)
+                 : "memory");
+}
+
+template <int RS, int L, int NCS>
+__global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
+    static_assert(L >= 1 && L <= 3, "blocks loaded ahead");
+    static_assert(NCS == 1 || NCS == 2 || NCS == 4, "copiers per step");
+    using C = DdscCfg<RS>;
+    using E = Elem<bf16_t>;
+    constexpr int NW = C::NW, NC = DC_NC;
+
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+    unsigned char* const a_ring = smem;
+    int* const s_items = reinterpret_cast<int*>(smem + C::ITEMS_OFF);
+    int* const s_steps = reinterpret_cast<int*>(smem + C::STEPS_OFF);
+    int* const s_landed = reinterpret_cast<int*>(smem + C::FLAG_OFF);   // [8]
+    int* const s_done = s_landed + NC;                                    // [16]
+    int* const s_fail = s_done + NW;
+    const unsigned lds_a = (unsigned)(uintptr_t)a_ring;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+#ifdef DC_PROF
+    const long long t_entry = (long long)__builtin_readcyclecounter();
+#endif
+
+    // Workgroup -> (column group, first token tile): the workgroups of one XCD cover all column groups of
+    // the same few token tiles, so a panel is fetched into that XCD's L2 once.
+    const int wg = blockIdx.x;
+#ifdef DC_MAP_GX
+    // experiment (8 groups, 32 workgroups per group): XCD x works on the groups 2 (x % 4), 2 (x % 4) + 1 only
+    const int xcd = wg & 7, slot = wg >> 3;
+    const int ng = 2 * (xcd & 3) + (slot & 1);
+    const int p = 2 * (slot >> 1) + (xcd >> 2);
+#elif defined(DC_MAP_G1)
+    // experiment: XCD x works on group x only
+    const int ng = wg & 7;
+    const int p = wg >> 3;
+#else
+    const int ng = (wg >> 3) % g.n_groups;
+    const int p = (wg & 7) + 8 * ((wg >> 3) / g.n_groups);
+#endif
+    if (p >= g.wg_per_group) return;
+    const int ntiles = (g.m_tiles - p + g.wg_per_group - 1) / g.wg_per_group;   // token tiles p, p + P, ...
+
+    const int KB = g.K / 32, KP = KB / 2;
+    const int* gplan = g.plan + (size_t)ng * g.group_ints;
+    // the header, one int per lane
+    const int v_hdr = gplan[lane];
+    const int ns = __builtin_amdgcn_readlane(v_hdr, 0);
+    const int my_col = __builtin_amdgcn_readlane(v_hdr, DC_H_COL + wave);
+    const bool has_col = my_col >= 0 && my_col * 32 < g.N;
+    const int ni = has_col ? __builtin_amdgcn_readlane(v_hdr, 1 + wave) : 0;
+    // items of the group -> LDS (column after column), or left in global memory when they do not fit
+    int ioff = 0, itotal = 0;
+#pragma unroll
+    for (int c = 0; c < NW; ++c) {
+        const int n = __builtin_amdgcn_readlane(v_hdr, 1 + c);
+        if (c < wave) ioff += n;
+        itotal += n;
+    }
+    const bool cached = itotal <= DC_ITEMS_LDS;
+    {
+        if (cached) {
+            int off = 0;
+#pragma unroll
+            for (int c = 0; c < NW; ++c) {
+                const int n = __builtin_amdgcn_readlane(v_hdr, 1 + c);
+                for (int i = tid; i < n; i += C::NT) s_items[off + i] = gplan[DC_HDR + KP + c * KB + i];
+                off += n;
+            }
+        }
+        for (int i = tid; i < ns; i += C::NT) s_steps[i] = gplan[DC_HDR + i];
+        if (tid < 64) s_landed[tid] = 0;   // landed, done, failure word
+    }
+    __syncthreads();
+    const int* g_items = gplan + DC_HDR + KP + wave * KB;
+    // 64 consecutive items of this wave's list, one per lane; single items are picked with v_readlane
+    auto items_window = [&](int win) __attribute__((always_inline)) -> int {
+        int i = win * 64 + lane;
+        if (i >= ni) i = 0;
+        int v;
+        if (cached) v = s_items[ioff + i];
+        else v = g_items[i];
+        asm volatile("" : "+v"(v));
+        return v;
+    };
+
+    const int nsteps = ns * ntiles;   // global steps of this workgroup (the host keeps this below 2^30)
+    const unsigned char* A = static_cast<const unsigned char*>(g.a);
+    const unsigned char* Dp = static_cast<const unsigned char*>(g.data);
+    const unsigned a_row_bytes = (unsigned)g.K * 2u;
+
+    // ---------------- copy side (waves NW - NC .. NW - 1) ----------------
+    const bool copier = wave >= NW - NC;
+    const int cidx = wave - (NW - NC);
+    constexpr int G = NC / NCS;              // groups of NCS copiers; group i copies the steps t with t % G == i
+    constexpr int CROWS = C::BM / NCS;       // rows of a step one copier copies
+    const int my_phase = (cidx / NCS) & (G - 1);
+    const int my_rows = (cidx % NCS) * CROWS;
+    const unsigned char* a_tile = A;
+    int a_last_row = 0;   // last valid row of the tile being copied (rows past the end re-read it; they are never stored)
+    auto enter_copy_tile = [&](int j) __attribute__((always_inline)) {
+        const int m0 = (p + j * g.wg_per_group) * C::BM;
+        a_last_row = g.M - 1 - m0;
+        a_tile = uniform_ptr(A + (size_t)m0 * a_row_bytes);
+    };
+    int t_mine = copier ? my_phase : nsteps, t_tile = 0, t_step = my_phase;   // next step this wave copies = step t_step of tile t_tile
+    while (t_step >= ns && ns > 0) {
+        t_step -= ns;
+        ++t_tile;
+    }
+    const unsigned landed_lds = (unsigned)(uintptr_t)(s_landed + (cidx & (NC - 1)));
+    bool gave_up = false;
+    int md = 0;            // last minimum of done[] seen (it only grows)
+
+    auto copy_step = [&]() __attribute__((always_inline)) {   // this wave's rows of step t_mine, then the number t_mine + 1 behind them
+        const int pair = __builtin_amdgcn_readfirstlane(s_steps[t_step]);
+        const unsigned char* src = uniform_ptr(a_tile + (size_t)pair * C::ROWB);
+        const unsigned stage = lds_a + ((unsigned)t_mine % (unsigned)RS) * C::PANEL_BYTES + (unsigned)my_rows * C::ROWB;
+        {
+            // lane l of instruction i: row my_rows + 8 i + l / 8, physical chunk l % 8 = logical chunk (l % 8) ^ swizzle(row)
+            int l = lane;
+            asm volatile("" : "+v"(l));
+#pragma unroll
+            for (int i = 0; i < CROWS / 8; ++i) {
+                const int row = my_rows + 8 * i + (l >> 3);
+                const int r = row < a_last_row ? row : a_last_row;
+                const unsigned voff = (unsigned)r * a_row_bytes + (unsigned)(((l & 7) ^ ((row >> 1) & 7)) * 16);
+#ifndef DC_ABL_NOPANELDMA
+                dma16(stage + i * 1024, src, voff);
+#else
+                asm volatile("" ::"v"(voff), "s"(src), "s"(stage));
+#endif
+            }
+        }
+#ifdef PBS_DDSC_PUBLISH_AFTER_WAIT
+        // checking build: wait for the rows, then write the number (relies on no ordering of one wave's loads)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (lane == 0) lds_poke(s_landed + cidx, t_mine + 1);
+#else
+        dma4_lane0(landed_lds, uniform_ptr(reinterpret_cast<const unsigned char*>(g.seq + (t_mine + 1))));
+#endif
+#ifdef DC_PROF_LAT
+        if (blockIdx.x == DC_PROF_WG && wave == DC_PROF_WAVE && t_mine / 2 < 500) {
+            // latency of this copy: spin until the progress word shows it
+            const long long t0 = (long long)__builtin_readcyclecounter();
+            int spins = 0;
+            while (__builtin_amdgcn_readfirstlane(lds_peek(s_landed + cidx)) != (t_mine + 1) && spins < 100000) ++spins;
+            const long long t1 = (long long)__builtin_readcyclecounter();
+            if (lane == 0) reinterpret_cast<long long*>(smem + C::LDS_BYTES)[1024 + t_mine / 2] = t1 - t0;
+        }
+#endif
+        t_mine += G;
+        t_step += G;
+        if (t_step >= ns) {
+            do {
+                t_step -= ns;
+                ++t_tile;
+            } while (t_step >= ns);
+            if (t_tile < ntiles) enter_copy_tile(t_tile);
+        }
+    };
+    // Copy this wave's steps whose ring slot is free according to the last done[] minimum seen; never waits.
+    auto try_copy = [&]() __attribute__((always_inline)) {
+        while (t_mine < nsteps && t_mine - RS < md) copy_step();
+    };
+
+    // ---------------- progress words ----------------
+    // One read: lanes 0..15 done[lane], the others the landed words of the NCS copiers of step u.
+    auto poll_issue = [&](int u) __attribute__((always_inline)) -> int {
+        int l = lane;
+        asm volatile("" : "+v"(l));
+        const int off = l < 16 ? (NC + l) * 4 : ((u & (G - 1)) * NCS + (l & (NCS - 1))) * 4;   // bytes from s_landed
+        return lds_peek(reinterpret_cast<const int*>(reinterpret_cast<const unsigned char*>(s_landed) + off));
+    };
+    // whether step u has landed: all of its copiers count at least u + 1 steps
+    auto poll_landed = [&](int v, int u) __attribute__((always_inline)) -> bool {
+        int m = __builtin_amdgcn_readlane(v, 16);
+#pragma unroll
+        for (int i = 1; i < NCS; ++i) {
+            const int w = __builtin_amdgcn_readlane(v, 16 + i);
+            m = w < m ? w : m;
+        }
+        return m > u;
+    };
+    // a copier also takes the minimum of done[] (-> md)
+    auto poll_done = [&](int v) __attribute__((always_inline)) {
+#define PBS_MIN_SHR(SH)                                                                \
+    {                                                                                  \
+        const int v2 = __builtin_amdgcn_update_dpp(v, v, 0x110 + SH, 0xf, 0xf, false); \
+        v = v2 < v ? v2 : v;                                                           \
+    }
+        PBS_MIN_SHR(1) PBS_MIN_SHR(2) PBS_MIN_SHR(4) PBS_MIN_SHR(8)
+#undef PBS_MIN_SHR
+        const int dmin = __builtin_amdgcn_readlane(v, 15);
+        md = dmin > md ? dmin : md;
+    };
+    auto publish_done = [&](int u) __attribute__((always_inline)) {
+        if (lane == 0) lds_poke(s_done + wave, u);
+    };
+    // wait until step u has landed, copying what becomes free meanwhile
+    auto slow_wait = [&](int u) __attribute__((always_inline)) {
+        bool here = false;
+        for (int spin = 0; spin < C::SPIN_LIMIT; ++spin) {
+            const int v = poll_issue(u);
+            here = poll_landed(v, u);
+            if (copier) {
+                poll_done(v);
+                try_copy();
+            }
+            if (here) break;
+            // another wave has given up: so does this one
+            if ((spin & 1023) == 1023 && __builtin_amdgcn_readfirstlane(lds_peek(s_fail)) != 0) break;
+            __builtin_amdgcn_s_sleep(DC_SLEEP);
+        }
+        if (!here) {
+            gave_up = true;
+            if (lane == 0) lds_poke(s_fail, 1);
+        }
+    };
+    // after the last item: copy this wave's remaining steps
+    auto copy_rest = [&]() __attribute__((always_inline)) {
+        for (int spin = 0; spin < C::SPIN_LIMIT && t_mine < nsteps && !gave_up; ++spin) {
+            const int before = md;
+            poll_done(poll_issue(0));
+            try_copy();
+            if (md != before) spin = 0;
+            if ((spin & 1023) == 1023 && __builtin_amdgcn_readfirstlane(lds_peek(s_fail)) != 0) break;
+            __builtin_amdgcn_s_sleep(DC_SLEEP);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    };
+
+    // ---------------- compute side ----------------
+    const int lrow = lane & 31;
+    const int h = lane >> 5;
+    // dense-operand fragment q of token slice t, k-block kk of a panel: 16 bytes at
+    //   (32 t + lrow) * 128 + ((4 kk + 2 q + h) ^ swizzle(lrow)) * 16  =  (a_pre ^ (64 kk + 32 q)) + 4096 t
+    const unsigned a_pre = (unsigned)(lrow * C::ROWB + ((h ^ ((lrow >> 1) & 7)) * 16));
+    // block fragment q: row lrow of the [n][k] block, 16 bytes at 16 (2 q + h)
+    const unsigned b_lane = (unsigned)(lrow * 64 + h * 16);
+
+    bf16_t* out = static_cast<bf16_t*>(g.out);
+    const bf16_t* bias = static_cast<const bf16_t*>(g.bias);
+
+    f32x16 acc[4];
+    auto zero_acc = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
+    };
+    zero_acc();
+
+    // Stores of one tile, straight from the accumulators.  Register quad q of a lane holds result columns
+    // 8 q + 4 h .. + 3 of token (lane % 32) of a slice.  The lane halves swap quads so that the lower half holds
+    // columns 8 q .. + 7 of quad q = 2 qq and the upper half those of quad q = 2 qq + 1: 16 contiguous bytes per lane.
+    auto epilogue = [&](int j) __attribute__((always_inline)) {
+        if (!has_col) return;
+        const int m0 = (p + j * g.wg_per_group) * C::BM;
+        const bool failed = gave_up || __builtin_amdgcn_readfirstlane(lds_peek(s_fail)) != 0;
+        int l = lane;
+        asm volatile("" : "+v"(l));
+        const int er = l & 31, eh = l >> 5;
+#pragma unroll
+        for (int qq = 0; qq < 2; ++qq) {
+            const int n0 = my_col * 32 + 8 * (2 * qq + eh);   // first of this lane's 8 result columns
+            uint4 braw = make_uint4(0u, 0u, 0u, 0u);
+            if (bias) braw = *reinterpret_cast<const uint4*>(bias + n0);
+            const uint32_t bw[4] = {braw.x, braw.y, braw.z, braw.w};
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                float x[8];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    // a = quad 2 qq (both halves), b = quad 2 qq + 1: after the swap a = [a lower, b lower], b = [a upper, b upper]
+                    const unsigned a = __float_as_uint(acc[t][4 * (2 * qq) + e]);
+                    const unsigned b = __float_as_uint(acc[t][4 * (2 * qq + 1) + e]);
+                    const auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+                    x[e] = __uint_as_float(r[0]);       // column 8 q' + e of this lane's quad q'
+                    x[4 + e] = __uint_as_float(r[1]);   // column 8 q' + 4 + e
+                }
+                uint32_t w[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float lo = x[2 * e] + __uint_as_float(bw[e] << 16);
+                    float hi = x[2 * e + 1] + __uint_as_float(bw[e] & 0xffff0000u);
+                    if (failed) lo = hi = __builtin_nanf("");
+                    w[e] = (uint32_t)E::from_f32(lo).bits | ((uint32_t)E::from_f32(hi).bits << 16);
+                }
+                const int row = m0 + t * 32 + er;
+                if (row < g.M) *reinterpret_cast<uint4*>(out + (size_t)row * g.N + n0) = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+        }
+    };
+
+    if (copier && ns > 0 && t_tile < ntiles) enter_copy_tile(t_tile);
+    if (ns == 0 || ni == 0) {
+        // nothing to multiply in this column: the wave only copies its share of the steps; its result columns are the bias
+        publish_done(0x7fffffff);
+        for (int j = 0; j < ntiles; ++j) epilogue(j);
+        if (ns > 0) copy_rest();
+        return;
+    }
+
+    const int total_items = ni * ntiles;
+    int vi_items = items_window(0), i_win = 0;   // the 64 items around the cursor
+    int vf_items = vi_items, f_win = 0;          // the 64 items around the block-load cursor
+    int j = 0, idx = 0;
+    int item = __builtin_amdgcn_readlane(vi_items, 0);
+    int u = item & 511;
+    publish_done(u);
+    // Block fragments: L + 1 register sets, item i uses set i % (L + 1); the block of item i + L is loaded while
+    // item i is worked on, into the set item i - 1 has just finished with.
+    u32x4 fb[L + 1][2];
+    int f_idx = 0;           // list index of the next item whose block is loaded
+    auto load_next_block = [&](u32x4& b0, u32x4& b1) __attribute__((always_inline)) {
+        if ((f_idx >> 6) != f_win) {
+            f_win = f_idx >> 6;
+            vf_items = items_window(f_win);
+        }
+        const unsigned id = (unsigned)__builtin_amdgcn_readlane(vf_items, f_idx & 63) >> 10;
+        // plain loads: the compiler places the wait before their first use (and never moves a register a load in
+        // flight is going to write)
+        const unsigned char* pb = Dp + ((size_t)id << 11) + b_lane;
+#ifndef DC_ABL_NOBLOCKLOAD
+        b0 = *reinterpret_cast<const u32x4*>(pb);
+        b1 = *reinterpret_cast<const u32x4*>(pb + 32);
+#else
+        b0 = b1 = u32x4{(unsigned)(uintptr_t)pb, 0u, 0u, 0u};
+#endif
+        if (++f_idx == ni) f_idx = 0;
+    };
+#pragma unroll
+    for (int i = 0; i < L; ++i) {
+        load_next_block(fb[i][0], fb[i][1]);
+    }
+    int raw = poll_issue(u);   // the progress words for the item a wave is about to start are read during the previous one
+
+#ifdef DC_PROF
+    long long* const s_prof = reinterpret_cast<long long*>(smem + C::LDS_BYTES);   // [1024][2]
+    const bool prof_on = blockIdx.x == DC_PROF_WG && wave == DC_PROF_WAVE;
+#define DC_T(k) do { if (prof_on && it < 600) { const long long tt = (long long)__builtin_readcyclecounter(); if (lane == 0) s_prof[it * 2 + (k)] = tt; } } while (0)
+#else
+#define DC_T(k) do { } while (0)
+#endif
+
+    // one item; S = the register set its block was loaded into; COPIER = this wave copies
+    auto do_item = [&](auto S_, auto COPIER_, int it) __attribute__((always_inline)) {
+        constexpr int S = decltype(S_)::value;
+        constexpr bool COPIER = decltype(COPIER_)::value;
+        constexpr int SF = (S + L) % (L + 1);
+        DC_T(0);
+        // has this item's step landed?
+        // (the read is always consumed: one left pending on one path costs a full wait at the join)
+        const bool here = poll_landed(raw, u);
+        if constexpr (COPIER) poll_done(raw);
+#ifndef DC_ABL_NOPANELWAIT
+        if (!here && !gave_up) slow_wait(u);   // after a failed wait nothing is waited for any more: the results are void
+#endif
+#ifdef DC_PROF
+        if (prof_on && it < 600) { const long long tt = (long long)__builtin_readcyclecounter(); if (lane == 0) s_prof[1200 + it] = tt; }   // time after the panel wait (shares the area: 3000 slots of 8 bytes = 24 KB)
+#endif
+        const int kk = (item >> 9) & 1;
+        // the next item
+        const bool more = it + 1 < total_items;
+        int idx_n = idx + 1, j_n = j;
+        if (idx_n == ni) {
+            idx_n = 0;
+            ++j_n;
+        }
+        if ((idx_n >> 6) != i_win) {
+            i_win = idx_n >> 6;
+            vi_items = items_window(i_win);
+        }
+        const int item_n = __builtin_amdgcn_readlane(vi_items, idx_n & 63);
+        const int u_n = more ? j_n * ns + (item_n & 511) : 0x7fffffff;
+        // the block of item it + L
+        // (always issued: behind the last item it re-reads a block of the list.  A load on one arm of a branch only
+        // would make the compiler wait for the worst case of both arms at the join.)
+        load_next_block(fb[SF][0], fb[SF][1]);
+        __builtin_amdgcn_sched_barrier(0);
+        // this item's dense-operand fragments, first half of k
+        const unsigned char* panel = a_ring + ((unsigned)u % (unsigned)RS) * C::PANEL_BYTES;
+        const unsigned off0 = a_pre ^ (unsigned)(kk * 64);
+        const unsigned char* pa0 = panel + off0;
+        const unsigned char* pa1 = panel + (off0 ^ 32u);
+        uint4 a0[4];
+#pragma unroll
+#ifndef DC_ABL_NOFRAGREAD
+        for (int t = 0; t < 4; ++t) a0[t] = *reinterpret_cast<const uint4*>(pa0 + t * 4096);
+#else
+        for (int t = 0; t < 4; ++t) a0[t] = make_uint4((unsigned)(uintptr_t)pa0, t, 0u, 0u);
+#endif
+        // the progress words for the next item, behind the fragment reads
+        raw = poll_issue(more ? u_n : 0);
+        if constexpr (COPIER) {
+            // The copy instructions are invisible to the compiler's count of outstanding loads, so its wait for this
+            // item's block also waits for as many older loads as copy instructions were issued since.  Issued here,
+            // right before that wait, they are the youngest: what the wait picks up instead are blocks loaded one or
+            // two items ago.
+            try_copy();
+        }
+        const bf16x8 w0 = __builtin_bit_cast(bf16x8, fb[S][0]);
+        const bf16x8 w1 = __builtin_bit_cast(bf16x8, fb[S][1]);
+#ifndef DC_ABL_NOMFMA
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w0, __builtin_bit_cast(bf16x8, a0[t]), acc[t], 0, 0, 0);
+#else
+#pragma unroll
+        for (int t = 0; t < 4; ++t) asm volatile("" ::"v"(fb[S][0]), "v"(a0[t].x), "v"(a0[t].w));
+#endif
+        // second half of k: fetched only now, into the registers the first half has left
+        __builtin_amdgcn_sched_barrier(0);
+        uint4 a1[4];
+#pragma unroll
+#ifndef DC_ABL_NOFRAGREAD
+        for (int t = 0; t < 4; ++t) a1[t] = *reinterpret_cast<const uint4*>(pa1 + t * 4096);
+#else
+        for (int t = 0; t < 4; ++t) a1[t] = make_uint4((unsigned)(uintptr_t)pa1, t, 0u, 0u);
+#endif
+        __builtin_amdgcn_sched_barrier(0);
+#ifndef DC_ABL_NOMFMA
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w1, __builtin_bit_cast(bf16x8, a1[t]), acc[t], 0, 0, 0);
+#else
+#pragma unroll
+        for (int t = 0; t < 4; ++t) asm volatile("" ::"v"(fb[S][1]), "v"(a1[t].x), "v"(a1[t].w));
+#endif
+        asm volatile("" ::: "memory");
+        if (u_n != u) publish_done(u_n);
+        DC_T(1);
+        if (j_n != j) {
+#ifdef DC_ABL_EPILAST
+            if (!more)
+#endif
+            epilogue(j);
+            zero_acc();
+        }
+        idx = idx_n;
+        j = j_n;
+        item = item_n;
+        u = u_n;
+    };
+    auto do_items = [&](auto self, auto S_, auto COPIER_, int it) __attribute__((always_inline)) -> void {
+        constexpr int S = decltype(S_)::value;
+        if (it < total_items) do_item(S_, COPIER_, it);
+        if constexpr (S < L) self(self, std::integral_constant<int, S + 1>{}, COPIER_, it + 1);
+    };
+    if (copier) {
+        for (int it = 0; it < total_items; it += L + 1) do_items(do_items, std::integral_constant<int, 0>{}, std::true_type{}, it);
+    } else {
+        for (int it = 0; it < total_items; it += L + 1) do_items(do_items, std::integral_constant<int, 0>{}, std::false_type{}, it);
+    }
+#ifdef DC_PROF
+    const long long t_items = (long long)__builtin_readcyclecounter();
+#endif
+    copy_rest();
+#ifdef DC_PROF
+    if (prof_on) {
+        const long long t_exit = (long long)__builtin_readcyclecounter();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        for (int i = lane; i < 1800; i += 64) g.prof[i < 1200 ? i : 2048 + (i - 1200)] = s_prof[i];
+#ifdef DC_PROF_LAT
+        for (int i = lane; i < 128; i += 64) g.prof[i] = reinterpret_cast<long long*>(smem + C::LDS_BYTES)[1024 + i];
+#endif
+        if (lane == 0) {
+            g.prof[2047] = t_exit;
+            g.prof[2046] = t_entry;
+            g.prof[2045] = total_items;
+            g.prof[2044] = ni;
+            g.prof[2043] = t_items;
+        }
+    }
+#endif
+}
+
+}  // namespace pbs
