@@ -44,6 +44,9 @@
 
 namespace pbs {
 
+#ifndef D16_SLEEP
+#define D16_SLEEP 1
+#endif
 constexpr int D16_NB = 16;      // block columns per tile
 constexpr int D16_REC = 64;     // ints per plan record
 constexpr int D16_F_PAIR = 32, D16_F_MASK = 33, D16_F_CUM = 34;
@@ -319,7 +322,7 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
                     free_now = true;
                     break;
                 }
-                __builtin_amdgcn_s_sleep(1);
+                __builtin_amdgcn_s_sleep(D16_SLEEP);
             }
             // Cannot happen unless the protocol is broken: say so; the compute waves mark their results.
             if (!free_now) lds_poke(s_fail, 1);
@@ -486,7 +489,7 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
                 for (int spin = 0; spin < C::SPIN_LIMIT; ++spin) {
                     landed = producers_landed(u);
                     if (landed > u) break;
-                    __builtin_amdgcn_s_sleep(1);
+                    __builtin_amdgcn_s_sleep(D16_SLEEP);
                 }
                 // Operands that never arrive mean a broken protocol, not a slow machine (a wave that is
                 // not running does not count polls).  Make the failure visible: the tiles become NaN.

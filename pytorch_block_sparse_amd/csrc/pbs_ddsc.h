@@ -4,7 +4,13 @@
 // block column of the tile for all 128 tokens: four 32 x 32 accumulators with fixed register names.
 // Its work is a list of items, one per stored block of its column, sorted by k; which accumulator a
 // product goes to never depends on the pattern, so the loop over items is straight-line code: 8 loads of
-// dense-operand fragments from LDS, 8 matrix instructions.  Four waves per SIMD cover each other's waits.
+// dense-operand fragments from LDS, 8 matrix instructions.
+//
+// What bounds this kernel is instruction issue: a SIMD issues at most one scalar, one vector, one LDS and one
+// vector-memory instruction per four cycles, shared by its four waves, so every bookkeeping instruction of an
+// item is paid several times over on the path of the wave with the most items.  Hence: everything that
+// depends on the pattern only is precomputed in the item words; a wave looks at one progress word per item;
+// waves that wait sleep long; only half of the waves copy.
 //
 // The block columns are ranked by block count and dealt to the waves so that every SIMD of every
 // workgroup gets the same number of blocks (ddsc_cols_kernel): places 0-3 of a group (one per SIMD) hold
@@ -13,15 +19,15 @@
 //
 // Operands.
 //   dense operand   A step is a pair of adjacent k-blocks (128-byte rows).  Its 128 x 64 panel goes
-//                   global -> LDS by DMA into a ring of RS steps (16 KB each).  Step t is copied by the four
-//                   waves 8 + 4 (t % 2) .. + 3, 32 rows = 4 DMA instructions each (a single wave cannot
-//                   issue DMA fast enough).
+//                   global -> LDS by DMA into a ring of RS steps (16 KB each).  Step t is copied by the
+//                   wave 8 + t % 8 (16 DMA instructions); eight copies are in flight at a time.
 //   packed blocks   never pass through LDS.  A block is multiplied by exactly one wave per token tile, so
 //                   the wave loads its two 16-byte fragments per lane straight from global memory into
-//                   registers, L items ahead.  That needs the block stored with k along its rows
-//                   ([n][k]); the stored layout is that for the input gradient, the forward product is
-//                   given a copy of the data with every block transposed (transpose_blocks_kernel).
-//   The LDS so freed makes the panel ring 8 or 9 steps deep, which covers the round trip of a DMA under load.
+//                   registers, DC_L items ahead, with ordinary loads (the compiler places the waits and never
+//                   moves a register a load in flight is going to write).  That needs the block stored with
+//                   k along its rows ([n][k]); the stored layout is that for the input gradient, the forward
+//                   product is given a copy of the data with every block transposed (transpose_blocks_kernel).
+//   The LDS so freed makes the panel ring 8 steps deep.
 //
 // The product is computed transposed, acc[n][token] (block fragment as first operand): a lane then holds
 // 4 consecutive result columns of one token per accumulator register quad; the two lane halves exchange
@@ -29,21 +35,21 @@
 // the registers.
 //
 // Progress words in LDS (one writer each, only growing; no barriers after the prologue):
-//   landed[c]   steps copied by copier c (wave 8 + c) whose rows have arrived, as (last step + 1) mod 256: behind
-//               its rows of step t the wave issues one single-lane 4-byte DMA that copies the number from a
-//               table in global memory onto the word; a wave's loads complete in order;
-//   done[w]     the global step wave w still needs: it has finished reading every earlier step.
-// Step t may overwrite ring slot t % RS once min done[] > t - RS.  Every step up to min landed[] - 2 has
-// arrived whatever its copiers; a wave remembers that bound and reads the words again only when its next
-// item lies beyond it.  A copier reads them for every item (it also needs min done[]), behind the item's
-// fragment reads, and reduces them after its matrix instructions, so the round trip is off the item's path.
-// Every wait polls with s_sleep and is bounded; a wait that runs into its bound (a broken protocol, not
-// a slow machine) makes the results NaN instead of passing silently.
+//   landed[c]   steps copied by copier c (wave 8 + c) whose rows have arrived (the number of the last one plus
+//               one): behind its rows of step t the wave issues one single-lane 4-byte DMA that copies the
+//               number from a table 0, 1, 2, ... in global memory onto the word; a wave's loads complete in order;
+//   done[w]     the global step wave w still needs: it has finished reading every earlier step (every lane
+//               writes its own copy of the word, lane 0's is read).
+// Step t may overwrite ring slot t % RS once min done[] > t - RS (the copiers poll that minimum); an item of
+// step u may be read when its copier's word exceeds u.  A wave reads that word for its next item behind the
+// current item's fragment reads and looks at it when it gets there, so the round trip is off the item's path.
+// Every wait polls with s_sleep and is bounded; a wait that runs into its bound (a broken protocol, not a slow
+// machine) makes the results NaN instead of passing silently.
 //
-// The block loads are ordinary loads: the compiler waits for them where their registers are first used.  It does
-// not see the DMA instructions (inline assembly), so in a copier such a wait covers as many older loads as DMA
-// instructions were issued since the block was requested; the DMA is therefore issued right before that
-// wait, where it is the youngest.  The heavy half issues no DMA and waits exactly.
+// The compiler does not see the DMA instructions (inline assembly), so in a copier its wait for a block
+// also covers as many older loads as DMA instructions were issued since the block was requested; the DMA
+// is therefore issued right before that wait, where it is the youngest.  The heavy half issues no DMA and
+// waits exactly.
 //
 // Persistent workgroups: a workgroup keeps one group of 16 block columns and walks several token
 // tiles; steps are numbered across tiles, so the first loads of a tile overlap the previous tile's stores.
@@ -51,8 +57,10 @@
 // Plan per group of 16 block columns (ddsc_plan_kernel), ints:
 //   [0] ns = k-pairs any column touches   [1 + c] items of column c   [17] 1 if the lists are usable
 //   [32 + c] block column of the result in place c (or -1)
-//   [64 + s]                  k-pair index of step s
-//   [64 + KP + c * KB + i]    item i of column c: step | (k & 1) << 9 | block << 10   (KP = K / 64, KB = K / 32)
+//   [64 + s]                          k-pair index of step s
+//   [64 + KP + 2 (c KB + i)]          item i of column c: step | (k & 1) << 9 | (1 << 10 if it is the column's last)
+//   [64 + KP + 2 (c KB + i) + 1]      byte offset in the data of the block of the column's item i + DC_L (cyclically)
+//   (KP = K / 64, KB = K / 32)
 #pragma once
 #include <type_traits>
 
@@ -62,17 +70,19 @@ namespace pbs {
 
 constexpr int DC_NB = 16;               // block columns per tile = waves per workgroup
 constexpr int DC_NC = 8;                // copiers: the waves DC_NB - DC_NC .. DC_NB - 1
+constexpr int DC_L = 2;                 // blocks loaded ahead of the item being multiplied
 constexpr int DC_BM = 128;              // tokens per tile
 constexpr int DC_HDR = 64;
 constexpr int DC_H_COL = 32;
 constexpr int DC_MAX_KP = 512;          // k-pairs (K <= 32768): 9 bits of an item
-constexpr int DC_MAX_BLOCKS = 1 << 21;  // block id: 22 bits of an item; byte offsets of blocks stay below 2^32
+constexpr int DC_ITEM_LAST = 1 << 10;
+constexpr int DC_MAX_BLOCKS = 1 << 21;  // byte offsets of blocks stay below 2^32
 constexpr int DC_ITEMS_LDS = 2048;      // items of a group kept in LDS (every pattern up to K = 4096)
 constexpr int DC_SEQ_INTS = 65536;      // the table 0, 1, 2, ...: a workgroup's steps are numbered below this
 #ifndef DC_SLEEP
-#define DC_SLEEP 2
+#define DC_SLEEP 8
 #endif
-static inline size_t ddsc_plan_group_ints(int KB) { return (size_t)DC_HDR + (KB / 2) + (size_t)DC_NB * KB; }
+static inline size_t ddsc_plan_group_ints(int KB) { return (size_t)DC_HDR + (KB / 2) + (size_t)DC_NB * 2 * KB; }
 
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
@@ -160,15 +170,18 @@ __global__ __launch_bounds__(256) void ddsc_plan_kernel(const int32_t* __restric
     __syncthreads();
     // items: thread c walks column c's entries (sorted by k; entries that are not are dropped)
     if (tid < DC_NB) {
-        int* items = out + DC_HDR + KP + (size_t)tid * KB;
+        int* items = out + DC_HDR + KP + (size_t)tid * 2 * KB;
         int n = 0, last = -1;
         for (int e = s_lo[tid]; e < s_hi[tid]; ++e) {
             const int kb = idx[2 * e], b = idx[2 * e + 1];
-            if (kb > last && kb < KB && b >= 0 && b < nnz) {
-                items[n++] = s_rank[kb >> 1] | ((kb & 1) << 9) | (b << 10);
+            if (kb > last && kb < KB && b >= 0 && b < nnz && b < DC_MAX_BLOCKS) {
+                items[2 * n] = s_rank[kb >> 1] | ((kb & 1) << 9);
+                items[2 * n + 1] = b;   // for now: the item's own block
+                ++n;
                 last = kb;
             }
         }
+        if (n > 0) items[2 * (n - 1)] |= DC_ITEM_LAST;
         out[1 + tid] = n;
     }
     if (tid == 0) {
@@ -179,6 +192,31 @@ __global__ __launch_bounds__(256) void ddsc_plan_kernel(const int32_t* __restric
     if (tid >= DC_H_COL + DC_NB && tid < DC_HDR) out[tid] = 0;
     // the numbers the waves publish their copies with
     for (int i = blockIdx.x * 256 + tid; i < DC_SEQ_INTS; i += gridDim.x * 256) seq[i] = i;
+}
+// Second pass over the plan: the second word of item i becomes the byte offset of the block of item i + DC_L (cyclically).
+// One workgroup per group; thread c does column c (in place: the rotation is done through a few registers).
+__global__ __launch_bounds__(64) void ddsc_plan_ahead_kernel(int KB, int* plan, int group_ints) {
+    const int tid = threadIdx.x;
+    if (tid >= DC_NB) return;
+    int* out = plan + (size_t)blockIdx.x * group_ints;
+    const int KP = KB / 2;
+    const int n = out[1 + tid];
+    if (n <= 0) return;
+    int* items = out + DC_HDR + KP + (size_t)tid * 2 * KB;
+    // the first DC_L blocks are needed again at the end
+    int first[DC_L];
+#pragma unroll
+    for (int i = 0; i < DC_L; ++i) first[i] = items[2 * (i % n) + 1];
+    for (int i = 0; i < n; ++i) {
+        const int src = i + DC_L;
+        int b;
+        if (src < n) b = items[2 * src + 1];
+        else {
+            const int r = (src - n) % n;   // wrapped: one of the first blocks (n may be smaller than DC_L)
+            b = r < DC_L ? first[r] : items[2 * r + 1];
+        }
+        items[2 * i + 1] = (int)((unsigned)b << 11);
+    }
 }
 
 // data_t block b = data block b transposed (32 x 32 elements of 2 bytes): one wave per block.
@@ -214,8 +252,8 @@ __global__ __launch_bounds__(256) void transpose_blocks_kernel(const uint16_t* _
 struct DdscArgs {
     const void* a;         // [M, K] row-major bf16
     const void* data;      // [nnz*32, 32] bf16, every block stored [n][k]
-    const int* plan;       // built by ddsc_plan_kernel for this pattern and direction
-    const int* seq;        // the table 0..255 written by ddsc_plan_kernel
+    const int* plan;       // built by ddsc_plan_kernel + ddsc_plan_ahead_kernel for this pattern and direction
+    const int* seq;        // the table 0, 1, 2, ... written by ddsc_plan_kernel
     const void* bias;      // nullptr or [N]
     void* out;             // [M, N] row-major
     int M, N, K, nnz;
@@ -232,12 +270,13 @@ struct DdscCfg {
     static constexpr int ROWB = 128;                   // one panel row: 64 k values
     static constexpr int PANEL_BYTES = BM * ROWB;      // 16 KB per step
     static constexpr int A_RING_BYTES = RS * PANEL_BYTES;
-    static constexpr int ITEMS_OFF = A_RING_BYTES;
-    static constexpr int STEPS_OFF = ITEMS_OFF + DC_ITEMS_LDS * 4;
-    static constexpr int FLAG_OFF = STEPS_OFF + DC_MAX_KP * 4;
-    static constexpr int LDS_BYTES = FLAG_OFF + 256;   // landed[8], done[16], failure word
+    static constexpr int ITEMS_OFF = A_RING_BYTES;                       // two words per item
+    static constexpr int STEPS_OFF = ITEMS_OFF + DC_ITEMS_LDS * 8;
+    static constexpr int DONE_OFF = STEPS_OFF + DC_MAX_KP * 4;           // done[16][64]
+    static constexpr int LANDED_OFF = DONE_OFF + NW * 256;               // landed[8], failure word
+    static constexpr int LDS_BYTES = LANDED_OFF + 256;
     static constexpr int SPIN_LIMIT = 1 << 18;
-    static_assert(RS >= 4 && RS <= 9, "ring depth");
+    static_assert(RS >= 4 && RS <= 8, "ring depth");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS");
 };
 
@@ -251,21 +290,20 @@ static __device__ __forceinline__ void dma4_lane0(unsigned lds_base_uniform, con
                  : "memory");
 }
 
-template <int RS, int L, int NCS>
+template <int RS, int NCS>
 __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
-    static_assert(L >= 1 && L <= 3, "blocks loaded ahead");
     static_assert(NCS == 1 || NCS == 2 || NCS == 4, "copiers per step");
     using C = DdscCfg<RS>;
     using E = Elem<bf16_t>;
-    constexpr int NW = C::NW, NC = DC_NC;
+    constexpr int NW = C::NW, NC = DC_NC, L = DC_L;
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
     unsigned char* const a_ring = smem;
     int* const s_items = reinterpret_cast<int*>(smem + C::ITEMS_OFF);
     int* const s_steps = reinterpret_cast<int*>(smem + C::STEPS_OFF);
-    int* const s_landed = reinterpret_cast<int*>(smem + C::FLAG_OFF);   // [8]
-    int* const s_done = s_landed + NC;                                    // [16]
-    int* const s_fail = s_done + NW;
+    int* const s_done = reinterpret_cast<int*>(smem + C::DONE_OFF);       // [16][64]
+    int* const s_landed = reinterpret_cast<int*>(smem + C::LANDED_OFF);   // [8]
+    int* const s_fail = s_landed + NC;
     const unsigned lds_a = (unsigned)(uintptr_t)a_ring;
 
     const int tid = threadIdx.x;
@@ -278,19 +316,8 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
     // Workgroup -> (column group, first token tile): the workgroups of one XCD cover all column groups of
     // the same few token tiles, so a panel is fetched into that XCD's L2 once.
     const int wg = blockIdx.x;
-#ifdef DC_MAP_GX
-    // experiment (8 groups, 32 workgroups per group): XCD x works on the groups 2 (x % 4), 2 (x % 4) + 1 only
-    const int xcd = wg & 7, slot = wg >> 3;
-    const int ng = 2 * (xcd & 3) + (slot & 1);
-    const int p = 2 * (slot >> 1) + (xcd >> 2);
-#elif defined(DC_MAP_G1)
-    // experiment: XCD x works on group x only
-    const int ng = wg & 7;
-    const int p = wg >> 3;
-#else
     const int ng = (wg >> 3) % g.n_groups;
     const int p = (wg & 7) + 8 * ((wg >> 3) / g.n_groups);
-#endif
     if (p >= g.wg_per_group) return;
     const int ntiles = (g.m_tiles - p + g.wg_per_group - 1) / g.wg_per_group;   // token tiles p, p + P, ...
 
@@ -302,42 +329,28 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
     const int my_col = __builtin_amdgcn_readlane(v_hdr, DC_H_COL + wave);
     const bool has_col = my_col >= 0 && my_col * 32 < g.N;
     const int ni = has_col ? __builtin_amdgcn_readlane(v_hdr, 1 + wave) : 0;
-    // items of the group -> LDS (column after column), or left in global memory when they do not fit
-    int ioff = 0, itotal = 0;
-#pragma unroll
-    for (int c = 0; c < NW; ++c) {
-        const int n = __builtin_amdgcn_readlane(v_hdr, 1 + c);
-        if (c < wave) ioff += n;
-        itotal += n;
-    }
-    const bool cached = itotal <= DC_ITEMS_LDS;
+    // items of the group -> LDS, column after column (the host launches this kernel only when they fit: K <= 4096)
+    int ioff = 0;
     {
-        if (cached) {
-            int off = 0;
+        int off = 0;
 #pragma unroll
-            for (int c = 0; c < NW; ++c) {
-                const int n = __builtin_amdgcn_readlane(v_hdr, 1 + c);
-                for (int i = tid; i < n; i += C::NT) s_items[off + i] = gplan[DC_HDR + KP + c * KB + i];
-                off += n;
-            }
+        for (int c = 0; c < NW; ++c) {
+            const int n = __builtin_amdgcn_readlane(v_hdr, 1 + c);
+            if (c == wave) ioff = off;
+            if (off + n <= DC_ITEMS_LDS)
+                for (int i = tid; i < 2 * n; i += C::NT) s_items[2 * off + i] = gplan[DC_HDR + KP + c * 2 * KB + i];
+            off += n;
         }
         for (int i = tid; i < ns; i += C::NT) s_steps[i] = gplan[DC_HDR + i];
-        if (tid < 64) s_landed[tid] = 0;   // landed, done, failure word
+        for (int i = tid; i < NW * 64 + 64; i += C::NT) s_done[i] = 0;   // done, landed, failure word
     }
     __syncthreads();
-    const int* g_items = gplan + DC_HDR + KP + wave * KB;
-    // 64 consecutive items of this wave's list, one per lane; single items are picked with v_readlane
-    auto items_window = [&](int win) __attribute__((always_inline)) -> int {
-        int i = win * 64 + lane;
-        if (i >= ni) i = 0;
-        int v;
-        if (cached) v = s_items[ioff + i];
-        else v = g_items[i];
-        asm volatile("" : "+v"(v));
-        return v;
+    const int* const my_items = s_items + 2 * ioff;
+    auto item_word = [&](int i, int w) __attribute__((always_inline)) -> int {   // word w of item i; every lane reads the same
+        return __builtin_amdgcn_readfirstlane(my_items[2 * i + w]);
     };
 
-    const int nsteps = ns * ntiles;   // global steps of this workgroup (the host keeps this below 2^30)
+    const int nsteps = ns * ntiles;   // global steps of this workgroup (the host keeps this below DC_SEQ_INTS)
     const unsigned char* A = static_cast<const unsigned char*>(g.a);
     const unsigned char* Dp = static_cast<const unsigned char*>(g.data);
     const unsigned a_row_bytes = (unsigned)g.K * 2u;
@@ -349,6 +362,9 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
     constexpr int CROWS = C::BM / NCS;       // rows of a step one copier copies
     const int my_phase = (cidx / NCS) & (G - 1);
     const int my_rows = (cidx % NCS) * CROWS;
+    // Lane l of DMA instruction i of a step: row my_rows + 8 i + l / 8, physical chunk l % 8 = logical chunk
+    // (l % 8) ^ ((row / 2) % 8).  my_rows is a multiple of 32, so the swizzle term is (l / 16) for even i and
+    // (l / 16) ^ 4 for odd i: two per-lane offsets serve all rows (the row advances in the scalar base address).
     const unsigned char* a_tile = A;
     int a_last_row = 0;   // last valid row of the tile being copied (rows past the end re-read it; they are never stored)
     auto enter_copy_tile = [&](int j) __attribute__((always_inline)) {
@@ -369,20 +385,34 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
         const int pair = __builtin_amdgcn_readfirstlane(s_steps[t_step]);
         const unsigned char* src = uniform_ptr(a_tile + (size_t)pair * C::ROWB);
         const unsigned stage = lds_a + ((unsigned)t_mine % (unsigned)RS) * C::PANEL_BYTES + (unsigned)my_rows * C::ROWB;
-        {
-            // lane l of instruction i: row my_rows + 8 i + l / 8, physical chunk l % 8 = logical chunk (l % 8) ^ swizzle(row)
-            int l = lane;
-            asm volatile("" : "+v"(l));
-#pragma unroll
-            for (int i = 0; i < CROWS / 8; ++i) {
-                const int row = my_rows + 8 * i + (l >> 3);
-                const int r = row < a_last_row ? row : a_last_row;
-                const unsigned voff = (unsigned)r * a_row_bytes + (unsigned)(((l & 7) ^ ((row >> 1) & 7)) * 16);
+        // (per-lane values are derived again from the lane id behind an opaque copy: kept across the item loop they
+        // would cost registers the accumulators and fragments need.  A rolled loop: this code must stay small.)
+        int lc = lane;
+        asm volatile("" : "+v"(lc));
+        const unsigned voff_row = (unsigned)(lc >> 3) * a_row_bytes;
+        const unsigned voff_even = voff_row + (unsigned)(((lc & 7) ^ (lc >> 4)) * 16);
+        const unsigned voff_odd = voff_row + (unsigned)(((lc & 7) ^ (lc >> 4) ^ 4) * 16);
+#pragma unroll 1
+        for (int i = 0; i < CROWS / 8; i += 2) {
+            const unsigned char* src_i = uniform_ptr(src + (size_t)(my_rows + 8 * i) * a_row_bytes);
+            if (my_rows + 8 * i + 15 <= a_last_row) {
+                // all 16 rows exist
 #ifndef DC_ABL_NOPANELDMA
-                dma16(stage + i * 1024, src, voff);
-#else
-                asm volatile("" ::"v"(voff), "s"(src), "s"(stage));
+                dma16(stage + i * 1024, src_i, voff_even);
+                dma16(stage + i * 1024 + 1024, src_i, voff_odd + 8u * a_row_bytes);
 #endif
+            } else {
+                // rows past the end of the matrix re-read its last row
+                const int l = lc;
+#pragma unroll
+                for (int ii = 0; ii < 2; ++ii) {
+                    const int row = my_rows + 8 * (i + ii) + (l >> 3);
+                    const int r = row < a_last_row ? row : a_last_row;   // row of the tile, never negative
+                    const unsigned voff = (unsigned)r * a_row_bytes + (unsigned)(((l & 7) ^ ((row >> 1) & 7)) * 16);
+#ifndef DC_ABL_NOPANELDMA
+                    dma16(stage + (i + ii) * 1024, src, voff);
+#endif
+                }
             }
         }
 #ifdef PBS_DDSC_PUBLISH_AFTER_WAIT
@@ -391,16 +421,6 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
         if (lane == 0) lds_poke(s_landed + cidx, t_mine + 1);
 #else
         dma4_lane0(landed_lds, uniform_ptr(reinterpret_cast<const unsigned char*>(g.seq + (t_mine + 1))));
-#endif
-#ifdef DC_PROF_LAT
-        if (blockIdx.x == DC_PROF_WG && wave == DC_PROF_WAVE && t_mine / 2 < 500) {
-            // latency of this copy: spin until the progress word shows it
-            const long long t0 = (long long)__builtin_readcyclecounter();
-            int spins = 0;
-            while (__builtin_amdgcn_readfirstlane(lds_peek(s_landed + cidx)) != (t_mine + 1) && spins < 100000) ++spins;
-            const long long t1 = (long long)__builtin_readcyclecounter();
-            if (lane == 0) reinterpret_cast<long long*>(smem + C::LDS_BYTES)[1024 + t_mine / 2] = t1 - t0;
-        }
 #endif
         t_mine += G;
         t_step += G;
@@ -418,11 +438,15 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
     };
 
     // ---------------- progress words ----------------
-    // One read: lanes 0..15 done[lane], the others the landed words of the NCS copiers of step u.
+    // One read: the landed word(s) of the NCS copiers of step u; a copier's lanes 0..15 read done[lane] instead.
     auto poll_issue = [&](int u) __attribute__((always_inline)) -> int {
-        int l = lane;
-        asm volatile("" : "+v"(l));
-        const int off = l < 16 ? (NC + l) * 4 : ((u & (G - 1)) * NCS + (l & (NCS - 1))) * 4;   // bytes from s_landed
+        int off = (u & (G - 1)) * NCS * 4;   // bytes from s_landed
+        if (NCS > 1 || copier) {
+            int l = lane;
+            asm volatile("" : "+v"(l));
+            if (NCS > 1) off += (l & (NCS - 1)) * 4;
+            if (copier) off = l < 16 ? l * 256 - NW * 256 : off;   // done[l] lies NW * 256 bytes before s_landed
+        }
         return lds_peek(reinterpret_cast<const int*>(reinterpret_cast<const unsigned char*>(s_landed) + off));
     };
     // whether step u has landed: all of its copiers count at least u + 1 steps
@@ -448,7 +472,9 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
         md = dmin > md ? dmin : md;
     };
     auto publish_done = [&](int u) __attribute__((always_inline)) {
-        if (lane == 0) lds_poke(s_done + wave, u);
+        int l = lane;
+        asm volatile("" : "+v"(l));
+        lds_poke(s_done + wave * 64 + l, u);
     };
     // wait until step u has landed, copying what becomes free meanwhile
     auto slow_wait = [&](int u) __attribute__((always_inline)) {
@@ -486,9 +512,10 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
     // ---------------- compute side ----------------
     const int lrow = lane & 31;
     const int h = lane >> 5;
-    // dense-operand fragment q of token slice t, k-block kk of a panel: 16 bytes at
-    //   (32 t + lrow) * 128 + ((4 kk + 2 q + h) ^ swizzle(lrow)) * 16  =  (a_pre ^ (64 kk + 32 q)) + 4096 t
-    const unsigned a_pre = (unsigned)(lrow * C::ROWB + ((h ^ ((lrow >> 1) & 7)) * 16));
+    // dense-operand fragment q of token slice t, k-block kk of the panel in ring slot s: 16 bytes at
+    //   16384 s + (32 t + lrow) * 128 + ((4 kk + 2 q + h) ^ swizzle(lrow)) * 16  =  (a_pre ^ (16384 s + 64 kk + 32 q)) + 4096 t
+    const unsigned a_pre = (unsigned)(lrow * C::ROWB + ((h ^ ((lrow >> 1) & 7)) * 16));   // offset within a_ring
+    static_assert((RS & (RS - 1)) == 0, "the ring slot is a bit field of the address");
     // block fragment q: row lrow of the [n][k] block, 16 bytes at 16 (2 q + h)
     const unsigned b_lane = (unsigned)(lrow * 64 + h * 16);
 
@@ -555,104 +582,101 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
         return;
     }
 
-    const int total_items = ni * ntiles;
-    int vi_items = items_window(0), i_win = 0;   // the 64 items around the cursor
-    int vf_items = vi_items, f_win = 0;          // the 64 items around the block-load cursor
-    int j = 0, idx = 0;
-    int item = __builtin_amdgcn_readlane(vi_items, 0);
-    int u = item & 511;
-    publish_done(u);
     // Block fragments: L + 1 register sets, item i uses set i % (L + 1); the block of item i + L is loaded while
     // item i is worked on, into the set item i - 1 has just finished with.
     u32x4 fb[L + 1][2];
-    int f_idx = 0;           // list index of the next item whose block is loaded
-    auto load_next_block = [&](u32x4& b0, u32x4& b1) __attribute__((always_inline)) {
-        if ((f_idx >> 6) != f_win) {
-            f_win = f_idx >> 6;
-            vf_items = items_window(f_win);
-        }
-        const unsigned id = (unsigned)__builtin_amdgcn_readlane(vf_items, f_idx & 63) >> 10;
-        // plain loads: the compiler places the wait before their first use (and never moves a register a load in
-        // flight is going to write)
-        const unsigned char* pb = Dp + ((size_t)id << 11) + b_lane;
+    auto load_block = [&](u32x4& b0, u32x4& b1, unsigned byte_off) __attribute__((always_inline)) {
+        // plain loads: the compiler places the wait before their first use
+        const unsigned char* pb = Dp + (size_t)(byte_off + b_lane);
 #ifndef DC_ABL_NOBLOCKLOAD
         b0 = *reinterpret_cast<const u32x4*>(pb);
         b1 = *reinterpret_cast<const u32x4*>(pb + 32);
 #else
         b0 = b1 = u32x4{(unsigned)(uintptr_t)pb, 0u, 0u, 0u};
 #endif
-        if (++f_idx == ni) f_idx = 0;
     };
+    // the blocks of the first L items: item i's block offset is the second word of item i - L (cyclically)
 #pragma unroll
     for (int i = 0; i < L; ++i) {
-        load_next_block(fb[i][0], fb[i][1]);
+        int src = (i - L) % ni;
+        if (src < 0) src += ni;
+        load_block(fb[i][0], fb[i][1], (unsigned)item_word(src, 1));
     }
+    // Items: 64 of them at a time sit in two registers (one per lane) and are picked with v_readlane; lists of more
+    // than 64 items are read from memory item by item.
+    const bool small = ni <= 64;
+    const int li = lane < ni ? lane : 0;
+    int vw0 = 0, vw1 = 0;
+    if (small) {
+        vw0 = my_items[2 * li];
+        vw1 = my_items[2 * li + 1];
+        asm volatile("" : "+v"(vw0), "+v"(vw1));
+    }
+    int idx = 0, j = 0;
+    int item = small ? __builtin_amdgcn_readlane(vw0, 0) : item_word(0, 0);
+    int u_base = 0;        // tile j's first global step
+    int u = item & 511;
+    publish_done(u);
     int raw = poll_issue(u);   // the progress words for the item a wave is about to start are read during the previous one
 
 #ifdef DC_PROF
-    long long* const s_prof = reinterpret_cast<long long*>(smem + C::LDS_BYTES);   // [1024][2]
+    long long* const s_prof = reinterpret_cast<long long*>(smem + C::LDS_BYTES);   // [300][2], then [300]
     const bool prof_on = blockIdx.x == DC_PROF_WG && wave == DC_PROF_WAVE;
-#define DC_T(k) do { if (prof_on && it < 600) { const long long tt = (long long)__builtin_readcyclecounter(); if (lane == 0) s_prof[it * 2 + (k)] = tt; } } while (0)
+    int it = 0;
+#define DC_T(k) do { if (prof_on && it < 300) { const long long tt = (long long)__builtin_readcyclecounter(); if (lane == 0) s_prof[it * 2 + (k)] = tt; } } while (0)
 #else
 #define DC_T(k) do { } while (0)
 #endif
 
-    // one item; S = the register set its block was loaded into; COPIER = this wave copies
-    auto do_item = [&](auto S_, auto COPIER_, int it) __attribute__((always_inline)) {
+    // one item; S = the register set its block was loaded into; COPIER = this wave copies; SMALL = the list is in registers
+    auto do_item = [&](auto S_, auto COPIER_, auto SMALL_) __attribute__((always_inline)) {
         constexpr int S = decltype(S_)::value;
         constexpr bool COPIER = decltype(COPIER_)::value;
+        constexpr bool SMALL = decltype(SMALL_)::value;
         constexpr int SF = (S + L) % (L + 1);
         DC_T(0);
-        // has this item's step landed?
-        // (the read is always consumed: one left pending on one path costs a full wait at the join)
+        // has this item's step landed?  (the read is always consumed: one left pending on one path costs a full wait at the join)
         const bool here = poll_landed(raw, u);
         if constexpr (COPIER) poll_done(raw);
 #ifndef DC_ABL_NOPANELWAIT
         if (!here && !gave_up) slow_wait(u);   // after a failed wait nothing is waited for any more: the results are void
 #endif
 #ifdef DC_PROF
-        if (prof_on && it < 600) { const long long tt = (long long)__builtin_readcyclecounter(); if (lane == 0) s_prof[1200 + it] = tt; }   // time after the panel wait (shares the area: 3000 slots of 8 bytes = 24 KB)
+        if (prof_on && it < 300) { const long long tt = (long long)__builtin_readcyclecounter(); if (lane == 0) s_prof[600 + it] = tt; }
 #endif
-        const int kk = (item >> 9) & 1;
-        // the next item
-        const bool more = it + 1 < total_items;
-        int idx_n = idx + 1, j_n = j;
-        if (idx_n == ni) {
-            idx_n = 0;
-            ++j_n;
+        // the block of item idx + L, and the next item (behind the last item of the last tile: the list's first again)
+        const bool last = (item & DC_ITEM_LAST) != 0;
+        const int idx_n = last ? 0 : idx + 1;
+        unsigned boff;
+        int item_n;
+        if constexpr (SMALL) {
+            boff = (unsigned)__builtin_amdgcn_readlane(vw1, idx);
+            item_n = __builtin_amdgcn_readlane(vw0, idx_n);
+        } else {
+            boff = (unsigned)item_word(idx, 1);
+            item_n = item_word(idx_n, 0);
         }
-        if ((idx_n >> 6) != i_win) {
-            i_win = idx_n >> 6;
-            vi_items = items_window(i_win);
-        }
-        const int item_n = __builtin_amdgcn_readlane(vi_items, idx_n & 63);
-        const int u_n = more ? j_n * ns + (item_n & 511) : 0x7fffffff;
-        // the block of item it + L
-        // (always issued: behind the last item it re-reads a block of the list.  A load on one arm of a branch only
-        // would make the compiler wait for the worst case of both arms at the join.)
-        load_next_block(fb[SF][0], fb[SF][1]);
+        const int u_base_n = last ? u_base + ns : u_base;
+        const int u_n = u_base_n + (item_n & 511);
+        load_block(fb[SF][0], fb[SF][1], boff);
         __builtin_amdgcn_sched_barrier(0);
         // this item's dense-operand fragments, first half of k
-        const unsigned char* panel = a_ring + ((unsigned)u % (unsigned)RS) * C::PANEL_BYTES;
-        const unsigned off0 = a_pre ^ (unsigned)(kk * 64);
-        const unsigned char* pa0 = panel + off0;
-        const unsigned char* pa1 = panel + (off0 ^ 32u);
+        const unsigned sel = ((unsigned)(u & (RS - 1)) << 14) | (unsigned)((item >> 3) & 64);   // ring slot, k-block of the pair
+        const unsigned ad0 = a_pre ^ sel, ad1 = ad0 ^ 32u;
+        // (pointers derived from the LDS array itself: an integer turned into a pointer would be a flat address)
+        const unsigned char* pa0 = a_ring + ad0;
+        const unsigned char* pa1 = a_ring + ad1;
         uint4 a0[4];
 #pragma unroll
 #ifndef DC_ABL_NOFRAGREAD
         for (int t = 0; t < 4; ++t) a0[t] = *reinterpret_cast<const uint4*>(pa0 + t * 4096);
 #else
-        for (int t = 0; t < 4; ++t) a0[t] = make_uint4((unsigned)(uintptr_t)pa0, t, 0u, 0u);
+        for (int t = 0; t < 4; ++t) a0[t] = make_uint4(ad0, t, 0u, 0u);
 #endif
         // the progress words for the next item, behind the fragment reads
-        raw = poll_issue(more ? u_n : 0);
-        if constexpr (COPIER) {
-            // The copy instructions are invisible to the compiler's count of outstanding loads, so its wait for this
-            // item's block also waits for as many older loads as copy instructions were issued since.  Issued here,
-            // right before that wait, they are the youngest: what the wait picks up instead are blocks loaded one or
-            // two items ago.
-            try_copy();
-        }
+        raw = poll_issue(u_n);
+        // (the copy instructions are issued here, right before the wait for this item's block, where they are the youngest)
+        if constexpr (COPIER) try_copy();
         const bf16x8 w0 = __builtin_bit_cast(bf16x8, fb[S][0]);
         const bf16x8 w1 = __builtin_bit_cast(bf16x8, fb[S][1]);
 #ifndef DC_ABL_NOMFMA
@@ -670,7 +694,7 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
 #ifndef DC_ABL_NOFRAGREAD
         for (int t = 0; t < 4; ++t) a1[t] = *reinterpret_cast<const uint4*>(pa1 + t * 4096);
 #else
-        for (int t = 0; t < 4; ++t) a1[t] = make_uint4((unsigned)(uintptr_t)pa1, t, 0u, 0u);
+        for (int t = 0; t < 4; ++t) a1[t] = make_uint4(ad1, t, 0u, 0u);
 #endif
         __builtin_amdgcn_sched_barrier(0);
 #ifndef DC_ABL_NOMFMA
@@ -682,30 +706,43 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
         for (int t = 0; t < 4; ++t) asm volatile("" ::"v"(fb[S][1]), "v"(a1[t].x), "v"(a1[t].w));
 #endif
         asm volatile("" ::: "memory");
-        if (u_n != u) publish_done(u_n);
+        publish_done(u_n);
         DC_T(1);
-        if (j_n != j) {
+        if (last) {
 #ifdef DC_ABL_EPILAST
-            if (!more)
+            if (j + 1 == ntiles)
 #endif
             epilogue(j);
             zero_acc();
+            ++j;
         }
         idx = idx_n;
-        j = j_n;
         item = item_n;
+        u_base = u_base_n;
         u = u_n;
+#ifdef DC_PROF
+        ++it;
+#endif
     };
-    auto do_items = [&](auto self, auto S_, auto COPIER_, int it) __attribute__((always_inline)) -> void {
-        constexpr int S = decltype(S_)::value;
-        if (it < total_items) do_item(S_, COPIER_, it);
-        if constexpr (S < L) self(self, std::integral_constant<int, S + 1>{}, COPIER_, it + 1);
+    auto run = [&](auto COPIER_, auto SMALL_) __attribute__((always_inline)) {
+        while (true) {
+            do_item(std::integral_constant<int, 0>{}, COPIER_, SMALL_);
+            if (j == ntiles) break;
+            do_item(std::integral_constant<int, 1>{}, COPIER_, SMALL_);
+            if (j == ntiles) break;
+            do_item(std::integral_constant<int, 2>{}, COPIER_, SMALL_);
+            if (j == ntiles) break;
+        }
     };
+    static_assert(L == 2, "the item loop is unrolled by L + 1 = 3");
     if (copier) {
-        for (int it = 0; it < total_items; it += L + 1) do_items(do_items, std::integral_constant<int, 0>{}, std::true_type{}, it);
+        if (small) run(std::true_type{}, std::true_type{});
+        else run(std::true_type{}, std::false_type{});
     } else {
-        for (int it = 0; it < total_items; it += L + 1) do_items(do_items, std::integral_constant<int, 0>{}, std::false_type{}, it);
+        if (small) run(std::false_type{}, std::true_type{});
+        else run(std::false_type{}, std::false_type{});
     }
+    publish_done(0x7fffffff);
 #ifdef DC_PROF
     const long long t_items = (long long)__builtin_readcyclecounter();
 #endif
@@ -714,14 +751,11 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
     if (prof_on) {
         const long long t_exit = (long long)__builtin_readcyclecounter();
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        for (int i = lane; i < 1800; i += 64) g.prof[i < 1200 ? i : 2048 + (i - 1200)] = s_prof[i];
-#ifdef DC_PROF_LAT
-        for (int i = lane; i < 128; i += 64) g.prof[i] = reinterpret_cast<long long*>(smem + C::LDS_BYTES)[1024 + i];
-#endif
+        for (int i = lane; i < 900; i += 64) g.prof[i < 600 ? i : 2048 + (i - 600)] = s_prof[i];
         if (lane == 0) {
             g.prof[2047] = t_exit;
             g.prof[2046] = t_entry;
-            g.prof[2045] = total_items;
+            g.prof[2045] = ni * ntiles;
             g.prof[2044] = ni;
             g.prof[2043] = t_items;
         }
