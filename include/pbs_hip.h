@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define PBS_ABI_VERSION 3
+#define PBS_ABI_VERSION 4
 #define PBS_BLOCK 32
 
 /* element type of dense operands, packed data and results (accumulation is fp32) */
@@ -103,6 +103,26 @@ int pbs_blocksparse_matmul(const void* dense_a, const void* data, const void* pl
                            const void* bias, void* dense_out,
                            int64_t tokens, int n, int k, int nnz,
                            int transpose, int dtype, void* stream);
+
+/*
+ * The same product with an optional workspace.  The reference's reverse_matmul_ hands its kernel a
+ * transposed copy of the packed data for one of the two directions, made on every call
+ * (block_sparse.py:541-544: data.reshape(-1, 32, 32).transpose(1, 2).reshape(-1, 32).contiguous()).
+ * The fastest bf16 kernel for patterns with many blocks per column wants the same for the forward
+ * direction (every block with the contraction index along its rows); the library makes that copy in
+ * `workspace`, on `stream`, before the product, when the caller provides one of
+ * pbs_blocksparse_matmul_workspace_bytes() bytes (16-byte aligned device memory, contents
+ * unspecified afterwards).  With workspace = NULL, or one that is too small, the call is
+ * pbs_blocksparse_matmul: same results to the last bit of bf16 rounding of the same fp32 sums in a
+ * different order, from a kernel that reads the data as stored.  ..._workspace_bytes() returns 0 when
+ * no workspace would be used (fp32, the input-gradient direction, small or very sparse problems).
+ */
+size_t pbs_blocksparse_matmul_workspace_bytes(int64_t tokens, int n, int k, int nnz, int transpose, int dtype);
+int pbs_blocksparse_matmul_ws(const void* dense_a, const void* data, const void* plan,
+                              const void* bias, void* dense_out,
+                              int64_t tokens, int n, int k, int nnz,
+                              int transpose, int dtype,
+                              void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * dense^T x dense -> block-sparse (only the nonzero blocks are computed), packed like

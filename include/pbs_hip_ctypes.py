@@ -27,6 +27,8 @@ PROTOTYPES = {
     "pbs_blocksparse_matmul_plan_bytes": (_z, [_i, _i]),
     "pbs_blocksparse_matmul_plan": (_i, [_p, _p, _i, _i, _i, _p, _z, _p]),
     "pbs_blocksparse_matmul": (_i, [_p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p]),
+    "pbs_blocksparse_matmul_workspace_bytes": (_z, [_l, _i, _i, _i, _i, _i]),
+    "pbs_blocksparse_matmul_ws": (_i, [_p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _z, _p]),
     "pbs_blocksparse_matmul_back_workspace_bytes": (_z, [_l, _i, _i, _i, _i]),
     "pbs_blocksparse_matmul_back": (_i, [_p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _p, _z, _p]),
 }
@@ -63,12 +65,15 @@ class PbsHip:
 
     def matmul(self, dense_a, data, plan, n, k, nnz, transpose, bias=None):
         """dense_a [tokens, k] row-major contiguous -> [tokens, n]; replaces the reference's call at block_sparse.py:562-574."""
-        out = torch.empty(dense_a.shape[0], n, dtype=dense_a.dtype, device=dense_a.device)
+        tokens, tr, dt = dense_a.shape[0], int(bool(transpose)), DTYPES[dense_a.dtype]
+        out = torch.empty(tokens, n, dtype=dense_a.dtype, device=dense_a.device)
+        # room for the transposed copy of the blocks that the reference makes itself at block_sparse.py:541-544
+        nws = self.lib.pbs_blocksparse_matmul_workspace_bytes(tokens, n, k, nnz, tr, dt)
+        ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=dense_a.device)
         with torch.cuda.device(dense_a.device):
-            self._check(self.lib.pbs_blocksparse_matmul(
+            self._check(self.lib.pbs_blocksparse_matmul_ws(
                 dense_a.data_ptr(), data.data_ptr(), plan.data_ptr(), None if bias is None else bias.data_ptr(),
-                out.data_ptr(), dense_a.shape[0], n, k, nnz, int(bool(transpose)), DTYPES[dense_a.dtype],
-                self._stream()), "matmul")
+                out.data_ptr(), tokens, n, k, nnz, tr, dt, ws.data_ptr(), nws, self._stream()), "matmul")
         return out
 
     def matmul_back(self, grad_out, inp, row_start_ends_a, cols_a, data_out):

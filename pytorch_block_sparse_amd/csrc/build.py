@@ -1,7 +1,7 @@
 """Compile libpbs_hip.so (the C-ABI HIP library) for gfx950 next to its sources.
 
-Also libpbs_hip_check.so: the same library with the wide bf16 kernel's conservative progress protocol
-(-DPBS_DDS16_PUBLISH_AFTER_WAIT).  Only tests/test_gpu_wide_protocol.py loads it, to compare the two bit for bit.
+Also libpbs_hip_check.so: the same library with the conservative progress protocol of the two barrier-free bf16
+kernels (-DPBS_DDS16_PUBLISH_AFTER_WAIT -DPBS_DDSC_PUBLISH_AFTER_WAIT).  Only tests/test_gpu_wide_protocol.py loads it, to compare the two bit for bit.
 """
 import os
 import subprocess
@@ -14,7 +14,7 @@ CHECK_LIB = os.path.join(HERE, "libpbs_hip_check.so")
 
 def build(verbose=True):
     _compile(LIB, [], verbose)
-    _compile(CHECK_LIB, ["-DPBS_DDS16_PUBLISH_AFTER_WAIT"], verbose)
+    _compile(CHECK_LIB, ["-DPBS_DDS16_PUBLISH_AFTER_WAIT", "-DPBS_DDSC_PUBLISH_AFTER_WAIT"], verbose)
     return LIB
 
 

@@ -62,16 +62,20 @@ static inline size_t dds_plan_group_ints(int KB) { return ((size_t)KB + 2) * DDS
 // tiles, for launches that would otherwise leave CUs without one.
 // slots[8g + j] = block column in place j of group g, or -1.  One workgroup.
 constexpr int DDS_BALANCE_MAX_COLS = 4096;
+constexpr int DDS_MIN_WIDTH = 5;   // the narrowest group the host asks for
+// places of all groups when DDS_BALANCE_MAX_COLS columns are dealt DDS_MIN_WIDTH to a group
+constexpr int DDS_SLOT_MAX = DDS_NB * ((DDS_BALANCE_MAX_COLS + DDS_MIN_WIDTH - 1) / DDS_MIN_WIDTH);
 __global__ __launch_bounds__(256) void dds_slots_kernel(const int32_t* __restrict__ ptr, int nblk_n, int n_groups,
                                                         int width, int* slots) {
     constexpr int NT = 256;
     __shared__ int s_cnt[DDS_BALANCE_MAX_COLS];
-    __shared__ int s_slot[DDS_BALANCE_MAX_COLS + DDS_NB];
+    __shared__ int s_slot[DDS_SLOT_MAX];
     __shared__ int s_max, s_sum;
     const int tid = threadIdx.x;
     const int total = n_groups * DDS_NB;
     bool skewed = false;
-    if (nblk_n <= DDS_BALANCE_MAX_COLS && n_groups >= 2) {
+    // (a table that would not fit s_slot keeps the natural order)
+    if (nblk_n <= DDS_BALANCE_MAX_COLS && n_groups >= 2 && total <= DDS_SLOT_MAX) {
         if (tid == 0) {
             s_max = 0;
             s_sum = 0;

@@ -78,7 +78,7 @@ constexpr int DC_MAX_KP = 512;          // k-pairs (K <= 32768): 9 bits of an it
 constexpr int DC_ITEM_LAST = 1 << 10;
 constexpr int DC_MAX_BLOCKS = 1 << 21;  // byte offsets of blocks stay below 2^32
 constexpr int DC_ITEMS_LDS = 2048;      // items of a group kept in LDS (every pattern up to K = 4096)
-constexpr int DC_SEQ_INTS = 65536;      // the table 0, 1, 2, ...: a workgroup's steps are numbered below this
+constexpr int DC_SEQ_INTS = 16384;      // the table 0, 1, 2, ...: a workgroup's steps are numbered below this
 #ifndef DC_SLEEP
 #define DC_SLEEP 8
 #endif
@@ -104,19 +104,25 @@ __global__ __launch_bounds__(256) void ddsc_cols_kernel(const int32_t* __restric
     for (int i = tid; i < total; i += NT) cols[i] = -1;
     for (int c = tid; c < nblk_n; c += NT) s_cnt[c] = clamp_entry(ptr[c + 1], nnz) - clamp_entry(ptr[c], nnz);
     __syncthreads();
-    const int units = 4 * n_groups;   // SIMD quarters: 4 places each
-    for (int c = tid; c < nblk_n; c += NT) {
-        const int n = s_cnt[c];
+    // Adjacent columns 2 q, 2 q + 1 stay together (places s and s + 4 of one group): their waves store the two halves
+    // of the same 128-byte lines of the result at about the same time, so the lines reach memory whole.
+    const int units = 4 * n_groups;   // SIMD quarters: 4 places = 2 pairs each
+    const int npairs = (nblk_n + 1) / 2;
+    for (int q = tid; q < npairs; q += NT) {
+        const int c0 = 2 * q, c1 = 2 * q + 1;
+        const int n = s_cnt[c0] + (c1 < nblk_n ? s_cnt[c1] : 0);
         int rank = 0;
-        for (int o = 0; o < nblk_n; ++o) {
-            const int m = s_cnt[o];
-            rank += (m > n || (m == n && o < c)) ? 1 : 0;
+        for (int o = 0; o < npairs; ++o) {
+            const int m = s_cnt[2 * o] + (2 * o + 1 < nblk_n ? s_cnt[2 * o + 1] : 0);
+            rank += (m > n || (m == n && o < q)) ? 1 : 0;
         }
-        const int turn = rank / units;             // 0..3: which of the quarter's 4 places
+        const int turn = rank / units;             // 0 or 1: which of the quarter's 2 pairs
         int u = rank % units;
-        if (turn & 1) u = units - 1 - u;           // serpentine: heavy and light columns pair up
-        // quarter u = (group u / 4, SIMD u % 4); its places are SIMD + 4 * turn
-        cols[(u >> 2) * DC_NB + (u & 3) + 4 * turn] = c;
+        if (turn & 1) u = units - 1 - u;           // serpentine: heavy and light pairs share a quarter
+        // quarter u = (group u / 4, SIMD u % 4); the pair's places are SIMD + 8 * turn and 4 more
+        const int place = (u >> 2) * DC_NB + (u & 3) + 8 * turn;
+        cols[place] = c0;
+        if (c1 < nblk_n) cols[place + 4] = c1;
     }
 }
 
@@ -259,9 +265,6 @@ struct DdscArgs {
     int M, N, K, nnz;
     int m_tiles, n_groups, group_ints;
     int wg_per_group;      // workgroups that share the token tiles of one column group
-#ifdef DC_PROF
-    long long* prof;
-#endif
 };
 
 template <int RS>
@@ -274,7 +277,8 @@ struct DdscCfg {
     static constexpr int STEPS_OFF = ITEMS_OFF + DC_ITEMS_LDS * 8;
     static constexpr int DONE_OFF = STEPS_OFF + DC_MAX_KP * 4;           // done[16][64]
     static constexpr int LANDED_OFF = DONE_OFF + NW * 256;               // landed[8], failure word
-    static constexpr int LDS_BYTES = LANDED_OFF + 256;
+    static constexpr int BIAS_OFF = LANDED_OFF + 256;                    // bias[16][32], 2 bytes each
+    static constexpr int LDS_BYTES = BIAS_OFF + NW * 64;
     static constexpr int SPIN_LIMIT = 1 << 18;
     static_assert(RS >= 4 && RS <= 8, "ring depth");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS");
@@ -309,9 +313,6 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-#ifdef DC_PROF
-    const long long t_entry = (long long)__builtin_readcyclecounter();
-#endif
 
     // Workgroup -> (column group, first token tile): the workgroups of one XCD cover all column groups of
     // the same few token tiles, so a panel is fetched into that XCD's L2 once.
@@ -343,6 +344,12 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
         }
         for (int i = tid; i < ns; i += C::NT) s_steps[i] = gplan[DC_HDR + i];
         for (int i = tid; i < NW * 64 + 64; i += C::NT) s_done[i] = 0;   // done, landed, failure word
+        // the bias of this wave's 32 result columns (zeros without one): the stores of a tile must not wait for a load
+        if (lane < 16) {
+            uint32_t b2 = 0u;
+            if (g.bias && has_col) b2 = reinterpret_cast<const uint32_t*>(static_cast<const bf16_t*>(g.bias) + my_col * 32)[lane];
+            reinterpret_cast<uint32_t*>(smem + C::BIAS_OFF)[wave * 16 + lane] = b2;
+        }
     }
     __syncthreads();
     const int* const my_items = s_items + 2 * ioff;
@@ -397,10 +404,8 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
             const unsigned char* src_i = uniform_ptr(src + (size_t)(my_rows + 8 * i) * a_row_bytes);
             if (my_rows + 8 * i + 15 <= a_last_row) {
                 // all 16 rows exist
-#ifndef DC_ABL_NOPANELDMA
                 dma16(stage + i * 1024, src_i, voff_even);
                 dma16(stage + i * 1024 + 1024, src_i, voff_odd + 8u * a_row_bytes);
-#endif
             } else {
                 // rows past the end of the matrix re-read its last row
                 const int l = lc;
@@ -409,9 +414,7 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
                     const int row = my_rows + 8 * (i + ii) + (l >> 3);
                     const int r = row < a_last_row ? row : a_last_row;   // row of the tile, never negative
                     const unsigned voff = (unsigned)r * a_row_bytes + (unsigned)(((l & 7) ^ ((row >> 1) & 7)) * 16);
-#ifndef DC_ABL_NOPANELDMA
                     dma16(stage + (i + ii) * 1024, src, voff);
-#endif
                 }
             }
         }
@@ -520,7 +523,6 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
     const unsigned b_lane = (unsigned)(lrow * 64 + h * 16);
 
     bf16_t* out = static_cast<bf16_t*>(g.out);
-    const bf16_t* bias = static_cast<const bf16_t*>(g.bias);
 
     f32x16 acc[4];
     auto zero_acc = [&]() __attribute__((always_inline)) {
@@ -544,8 +546,7 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
 #pragma unroll
         for (int qq = 0; qq < 2; ++qq) {
             const int n0 = my_col * 32 + 8 * (2 * qq + eh);   // first of this lane's 8 result columns
-            uint4 braw = make_uint4(0u, 0u, 0u, 0u);
-            if (bias) braw = *reinterpret_cast<const uint4*>(bias + n0);
+            const uint4 braw = *reinterpret_cast<const uint4*>(smem + C::BIAS_OFF + wave * 64 + 16 * (2 * qq + eh));
             const uint32_t bw[4] = {braw.x, braw.y, braw.z, braw.w};
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
@@ -588,12 +589,8 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
     auto load_block = [&](u32x4& b0, u32x4& b1, unsigned byte_off) __attribute__((always_inline)) {
         // plain loads: the compiler places the wait before their first use
         const unsigned char* pb = Dp + (size_t)(byte_off + b_lane);
-#ifndef DC_ABL_NOBLOCKLOAD
         b0 = *reinterpret_cast<const u32x4*>(pb);
         b1 = *reinterpret_cast<const u32x4*>(pb + 32);
-#else
-        b0 = b1 = u32x4{(unsigned)(uintptr_t)pb, 0u, 0u, 0u};
-#endif
     };
     // the blocks of the first L items: item i's block offset is the second word of item i - L (cyclically)
 #pragma unroll
@@ -619,14 +616,6 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
     publish_done(u);
     int raw = poll_issue(u);   // the progress words for the item a wave is about to start are read during the previous one
 
-#ifdef DC_PROF
-    long long* const s_prof = reinterpret_cast<long long*>(smem + C::LDS_BYTES);   // [300][2], then [300]
-    const bool prof_on = blockIdx.x == DC_PROF_WG && wave == DC_PROF_WAVE;
-    int it = 0;
-#define DC_T(k) do { if (prof_on && it < 300) { const long long tt = (long long)__builtin_readcyclecounter(); if (lane == 0) s_prof[it * 2 + (k)] = tt; } } while (0)
-#else
-#define DC_T(k) do { } while (0)
-#endif
 
     // one item; S = the register set its block was loaded into; COPIER = this wave copies; SMALL = the list is in registers
     auto do_item = [&](auto S_, auto COPIER_, auto SMALL_) __attribute__((always_inline)) {
@@ -634,16 +623,10 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
         constexpr bool COPIER = decltype(COPIER_)::value;
         constexpr bool SMALL = decltype(SMALL_)::value;
         constexpr int SF = (S + L) % (L + 1);
-        DC_T(0);
         // has this item's step landed?  (the read is always consumed: one left pending on one path costs a full wait at the join)
         const bool here = poll_landed(raw, u);
         if constexpr (COPIER) poll_done(raw);
-#ifndef DC_ABL_NOPANELWAIT
         if (!here && !gave_up) slow_wait(u);   // after a failed wait nothing is waited for any more: the results are void
-#endif
-#ifdef DC_PROF
-        if (prof_on && it < 300) { const long long tt = (long long)__builtin_readcyclecounter(); if (lane == 0) s_prof[600 + it] = tt; }
-#endif
         // the block of item idx + L, and the next item (behind the last item of the last tile: the list's first again)
         const bool last = (item & DC_ITEM_LAST) != 0;
         const int idx_n = last ? 0 : idx + 1;
@@ -668,50 +651,28 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
         const unsigned char* pa1 = a_ring + ad1;
         uint4 a0[4];
 #pragma unroll
-#ifndef DC_ABL_NOFRAGREAD
         for (int t = 0; t < 4; ++t) a0[t] = *reinterpret_cast<const uint4*>(pa0 + t * 4096);
-#else
-        for (int t = 0; t < 4; ++t) a0[t] = make_uint4(ad0, t, 0u, 0u);
-#endif
         // the progress words for the next item, behind the fragment reads
         raw = poll_issue(u_n);
         // (the copy instructions are issued here, right before the wait for this item's block, where they are the youngest)
         if constexpr (COPIER) try_copy();
         const bf16x8 w0 = __builtin_bit_cast(bf16x8, fb[S][0]);
         const bf16x8 w1 = __builtin_bit_cast(bf16x8, fb[S][1]);
-#ifndef DC_ABL_NOMFMA
 #pragma unroll
         for (int t = 0; t < 4; ++t)
             acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w0, __builtin_bit_cast(bf16x8, a0[t]), acc[t], 0, 0, 0);
-#else
-#pragma unroll
-        for (int t = 0; t < 4; ++t) asm volatile("" ::"v"(fb[S][0]), "v"(a0[t].x), "v"(a0[t].w));
-#endif
         // second half of k: fetched only now, into the registers the first half has left
         __builtin_amdgcn_sched_barrier(0);
         uint4 a1[4];
 #pragma unroll
-#ifndef DC_ABL_NOFRAGREAD
         for (int t = 0; t < 4; ++t) a1[t] = *reinterpret_cast<const uint4*>(pa1 + t * 4096);
-#else
-        for (int t = 0; t < 4; ++t) a1[t] = make_uint4(ad1, t, 0u, 0u);
-#endif
         __builtin_amdgcn_sched_barrier(0);
-#ifndef DC_ABL_NOMFMA
 #pragma unroll
         for (int t = 0; t < 4; ++t)
             acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w1, __builtin_bit_cast(bf16x8, a1[t]), acc[t], 0, 0, 0);
-#else
-#pragma unroll
-        for (int t = 0; t < 4; ++t) asm volatile("" ::"v"(fb[S][1]), "v"(a1[t].x), "v"(a1[t].w));
-#endif
         asm volatile("" ::: "memory");
         publish_done(u_n);
-        DC_T(1);
         if (last) {
-#ifdef DC_ABL_EPILAST
-            if (j + 1 == ntiles)
-#endif
             epilogue(j);
             zero_acc();
             ++j;
@@ -720,9 +681,6 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
         item = item_n;
         u_base = u_base_n;
         u = u_n;
-#ifdef DC_PROF
-        ++it;
-#endif
     };
     auto run = [&](auto COPIER_, auto SMALL_) __attribute__((always_inline)) {
         while (true) {
@@ -743,24 +701,7 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
         else run(std::false_type{}, std::false_type{});
     }
     publish_done(0x7fffffff);
-#ifdef DC_PROF
-    const long long t_items = (long long)__builtin_readcyclecounter();
-#endif
     copy_rest();
-#ifdef DC_PROF
-    if (prof_on) {
-        const long long t_exit = (long long)__builtin_readcyclecounter();
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        for (int i = lane; i < 900; i += 64) g.prof[i < 600 ? i : 2048 + (i - 600)] = s_prof[i];
-        if (lane == 0) {
-            g.prof[2047] = t_exit;
-            g.prof[2046] = t_entry;
-            g.prof[2045] = ni * ntiles;
-            g.prof[2044] = ni;
-            g.prof[2043] = t_items;
-        }
-    }
-#endif
 }
 
 }  // namespace pbs

@@ -5,11 +5,13 @@
 
 #include <atomic>
 #include <cmath>
+#include <cstdlib>
 #include <mutex>
 
 #include "pbs_common.h"
 #include "pbs_dds.h"
 #include "pbs_dds16.h"
+#include "pbs_ddsc.h"
 #include "pbs_index.h"
 #include "pbs_sdd.h"
 #include "pbs_sdd_bf16.h"
@@ -65,6 +67,7 @@ static int launch_dds(DdsArgs g, hipStream_t stream) {
 // token count, which is not known when the plan is built.
 constexpr int DDS_NWIDTHS = 4;
 constexpr int DDS_WIDTHS[DDS_NWIDTHS] = {8, 7, 6, 5};
+static_assert(DDS_WIDTHS[DDS_NWIDTHS - 1] == DDS_MIN_WIDTH, "dds_slots_kernel sizes its table for the narrowest group");
 static inline size_t narrow_groups(int n, int wi) { return ((size_t)(n / 32) + DDS_WIDTHS[wi] - 1) / DDS_WIDTHS[wi]; }
 static inline size_t narrow_plan_bytes_w(int n, int k, int wi) {
     return narrow_groups(n, wi) * dds_plan_group_ints(k / 32) * sizeof(int);
@@ -92,12 +95,23 @@ static inline size_t slot_table_offset(int n, int k, int wi) {
     if (wi == 0) return narrow_plan_bytes(n, k) + wide_plan_bytes(n, k);
     return narrow_plan_offset(n, k, wi) + narrow_plan_bytes_w(n, k, wi);
 }
-static inline size_t all_plan_bytes(int n, int k) {
+// ... and behind all of those the plan of the kernel with one block column per wave (pbs_ddsc.h), where it can
+// apply: [column table][per-group lists][the table 0, 1, 2, ...].
+static inline size_t column_plan_offset(int n, int k) {
     return narrow_plan_offset(n, k, DDS_NWIDTHS - 1) + narrow_plan_bytes_w(n, k, DDS_NWIDTHS - 1) +
            slot_table_bytes_w(n, DDS_NWIDTHS - 1);
 }
+static inline int column_groups(int n) { return (n / 32 + DC_NB - 1) / DC_NB; }
+static inline size_t column_table_bytes(int n) { return ((size_t)column_groups(n) * DC_NB * sizeof(int) + 63) / 64 * 64; }
+static inline size_t column_plan_bytes(int n, int k) {
+    // k-pairs, and the lists of a group of 16 columns must fit the kernel's LDS area (16 * k / 32 items)
+    if ((k % 64) || DC_NB * (k / 32) > DC_ITEMS_LDS) return 0;
+    return column_table_bytes(n) + ((size_t)column_groups(n) * ddsc_plan_group_ints(k / 32) + DC_SEQ_INTS) * sizeof(int);
+}
+static inline size_t all_plan_bytes(int n, int k) { return column_plan_offset(n, k) + column_plan_bytes(n, k); }
 
 constexpr int D16_TM = 2, D16_RS = 3, D16_RB = 32, D16_NP = 4;
+constexpr double DDSC_MIN_BLOCKS_PER_COLUMN = 40.0;
 
 // Whether the wide kernel serves this problem: k-pairs need k % 64 == 0, the plan records of a group
 // must fit in LDS beside the rings, and there must be enough tiles to give every CU one.
@@ -142,6 +156,73 @@ static int launch_dds16(const DdsArgs& g, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
+// ---- bf16 kernel with one block column per wave ----
+constexpr int DDSC_RS = 8, DDSC_NCS = 1;
+
+// PBS_COLUMN_KERNEL = 0: never use it; 1: whenever it can run; unset: where it is the faster one.
+static int column_kernel_wish() {
+    const char* e = std::getenv("PBS_COLUMN_KERNEL");
+    if (!e || !*e) return -1;
+    return e[0] == '0' ? 0 : 1;
+}
+
+struct ColumnLaunch {
+    int m_tiles, n_groups, wg_per_group;
+};
+static inline ColumnLaunch column_launch(long long M, int n) {
+    ColumnLaunch c;
+    c.m_tiles = (int)((M + DC_BM - 1) / DC_BM);
+    c.n_groups = column_groups(n);
+    int P = 256 / c.n_groups;   // about one workgroup per CU, each walking the token tiles p, p + P, ... of its column group
+    if (P < 1) P = 1;
+    if (P > c.m_tiles) P = c.m_tiles;
+    c.wg_per_group = P;
+    return c;
+}
+
+// Whether that kernel can run this problem at all, and whether it should.  It reads a block's fragments straight
+// from global memory, once per token tile, and pays per step (one k-pair of one tile) what the wide kernel pays,
+// so it wins where the steps are long: many blocks per column.
+static bool column_kernel_fits(long long M, int n, int k, int nnz, const void* bias) {
+    if (!column_plan_bytes(n, k) || nnz < 1 || nnz > DC_MAX_BLOCKS || M < 1) return false;
+    if (reinterpret_cast<uintptr_t>(bias) & 3u) return false;
+    const ColumnLaunch c = column_launch(M, n);
+    const long long tiles_per_wg = (c.m_tiles + c.wg_per_group - 1) / c.wg_per_group;
+    if (tiles_per_wg * (k / 64) >= DC_SEQ_INTS) return false;   // a workgroup's steps are numbered through the table
+    const int wish = column_kernel_wish();
+    if (wish >= 0) return wish == 1;
+    if ((long long)c.m_tiles * c.n_groups < 256) return false;
+    return (double)nnz / (n / 32) >= DDSC_MIN_BLOCKS_PER_COLUMN;
+}
+
+static int launch_ddsc(const DdsArgs& g, const void* data_nk, hipStream_t stream) {
+    using C = DdscCfg<DDSC_RS>;
+    static std::atomic<uint64_t> done{0};
+    auto kernel = ddsc_kernel<DDSC_RS, DDSC_NCS>;
+    const ColumnLaunch c = column_launch(g.M, g.N);
+    DdscArgs a;
+    a.a = g.a;
+    a.data = data_nk;
+    a.plan = reinterpret_cast<const int*>(reinterpret_cast<const unsigned char*>(g.plan) + column_plan_offset(g.N, g.K) +
+                                          column_table_bytes(g.N));
+    a.bias = g.bias;
+    a.out = g.out;
+    a.M = g.M;
+    a.N = g.N;
+    a.K = g.K;
+    a.nnz = g.nnz;
+    a.m_tiles = c.m_tiles;
+    a.n_groups = c.n_groups;
+    a.group_ints = (int)ddsc_plan_group_ints(g.K / 32);
+    a.seq = a.plan + (size_t)a.n_groups * a.group_ints;
+    a.wg_per_group = c.wg_per_group;
+    if (int rc = raise_lds_limit(kernel, 160 * 1024, done)) return rc;
+    const long long grid = 8ll * a.n_groups * ((c.wg_per_group + 7) / 8);
+    if (grid > (1ll << 30)) return PBS_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(C::NT), C::LDS_BYTES, stream, a);
+    return (int)hipGetLastError();
+}
+
 // Tile shapes: 256 tokens x 8 block columns, 128 x 8, or 128 x 4 (twice as many, half as wide tiles).
 // One workgroup runs per CU, so a launch takes ceil(tiles / 256) rounds of one tile time each; the shape
 // with the smallest rounds x tile area wins (smaller tiles move more operand bytes per product, hence the
@@ -150,8 +231,19 @@ static int launch_dds16(const DdsArgs& g, hipStream_t stream) {
 // rings and plan records do not fit in LDS (very long contractions) is skipped.
 // bf16 steps cover two k-blocks (the matrix cores go through a k-block 16x faster than in fp32).
 template <typename T, int TRANS>
-static int dispatch_dds(const DdsArgs& g, hipStream_t stream) {
+static int dispatch_dds(const DdsArgs& g, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     if constexpr (sizeof(T) == 2) {
+        if (column_kernel_fits(g.M, g.N, g.K, g.nnz, g.bias)) {
+            // the kernel wants every block with k along its rows: as stored for TRANS, a transposed copy otherwise
+            if constexpr (TRANS) return launch_ddsc(g, g.data, stream);
+            const size_t need = (size_t)g.nnz * 2048;
+            if (workspace && workspace_bytes >= need && aligned16(workspace)) {
+                hipLaunchKernelGGL(transpose_blocks_kernel, dim3((unsigned)((g.nnz + 3) / 4)), dim3(256), 0, stream,
+                                   static_cast<const uint16_t*>(g.data), static_cast<uint16_t*>(workspace), g.nnz);
+                if (int rc = (int)hipGetLastError()) return rc;
+                return launch_ddsc(g, workspace, stream);
+            }
+        }
         if (wide_kernel_fits(g.M, g.N, g.K)) return launch_dds16<TRANS>(g, stream);
     }
     // shapes: 0 = 256 x 8 (4 token slices x 2 column halves), 1 = 128 x 8, 2 = 128 x 4,
@@ -498,12 +590,39 @@ int pbs_blocksparse_matmul_plan(const int32_t* ptr, const int32_t* indices, int 
         hipLaunchKernelGGL(dds16_plan_kernel, dim3(groups16), dim3(256), 0, static_cast<hipStream_t>(stream), ptr, indices,
                            n / 32, k / 32, nnz, wide, (int)dds16_plan_group_ints(k / 32),
                            wide + (size_t)groups16 * dds16_plan_group_ints(k / 32));
+        if (int rc = (int)hipGetLastError()) return rc;
+    }
+    if (column_plan_bytes(n, k)) {
+        const int groups = column_groups(n);
+        const int group_ints = (int)ddsc_plan_group_ints(k / 32);
+        int* cols = reinterpret_cast<int*>(static_cast<unsigned char*>(plan) + column_plan_offset(n, k));
+        int* lists = reinterpret_cast<int*>(static_cast<unsigned char*>(plan) + column_plan_offset(n, k) + column_table_bytes(n));
+        hipStream_t s = static_cast<hipStream_t>(stream);
+        hipLaunchKernelGGL(ddsc_cols_kernel, dim3(1), dim3(256), 0, s, ptr, n / 32, groups, nnz, cols);
+        if (int rc = (int)hipGetLastError()) return rc;
+        hipLaunchKernelGGL(ddsc_plan_kernel, dim3(groups), dim3(256), 0, s, ptr, indices, cols, n / 32, k / 32, nnz, lists,
+                           group_ints, lists + (size_t)groups * group_ints);
+        if (int rc = (int)hipGetLastError()) return rc;
+        hipLaunchKernelGGL(ddsc_plan_ahead_kernel, dim3(groups), dim3(64), 0, s, k / 32, lists, group_ints);
     }
     return (int)hipGetLastError();
 }
 
+size_t pbs_blocksparse_matmul_workspace_bytes(int64_t tokens, int n, int k, int nnz, int transpose, int dtype) {
+    if (dtype != PBS_DTYPE_BF16 || !transpose || tokens <= 0 || n <= 0 || k <= 0 || nnz <= 0 || (n % 32) || (k % 32)) return 0;
+    if ((long long)nnz > (long long)(n / 32) * (k / 32)) return 0;
+    return column_kernel_fits(tokens, n, k, nnz, nullptr) ? (size_t)nnz * 2048 : 0;
+}
+
 int pbs_blocksparse_matmul(const void* dense_a, const void* data, const void* plan, const void* bias, void* dense_out,
                            int64_t tokens, int n, int k, int nnz, int transpose, int dtype, void* stream) {
+    return pbs_blocksparse_matmul_ws(dense_a, data, plan, bias, dense_out, tokens, n, k, nnz, transpose, dtype, nullptr, 0,
+                                     stream);
+}
+
+int pbs_blocksparse_matmul_ws(const void* dense_a, const void* data, const void* plan, const void* bias, void* dense_out,
+                              int64_t tokens, int n, int k, int nnz, int transpose, int dtype, void* workspace,
+                              size_t workspace_bytes, void* stream) {
     if (dtype != PBS_DTYPE_F32 && dtype != PBS_DTYPE_BF16) return PBS_ERR_BAD_DTYPE;
     if (tokens < 0 || n <= 0 || k <= 0 || nnz < 0 || (n % 32) || (k % 32)) return PBS_ERR_BAD_SHAPE;
     if (tokens > (1ll << 30) || (long long)nnz > (long long)(n / 32) * (k / 32) || k > (1 << 24)) return PBS_ERR_TOO_LARGE;
@@ -526,9 +645,10 @@ int pbs_blocksparse_matmul(const void* dense_a, const void* data, const void* pl
     g.group_ints = (int)dds_plan_group_ints(k / 32);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == PBS_DTYPE_F32) {
-        return transpose ? dispatch_dds<float, 0>(g, s) : dispatch_dds<float, 1>(g, s);
+        return transpose ? dispatch_dds<float, 0>(g, nullptr, 0, s) : dispatch_dds<float, 1>(g, nullptr, 0, s);
     }
-    return transpose ? dispatch_dds<bf16_t, 0>(g, s) : dispatch_dds<bf16_t, 1>(g, s);
+    return transpose ? dispatch_dds<bf16_t, 0>(g, workspace, workspace_bytes, s)
+                     : dispatch_dds<bf16_t, 1>(g, nullptr, 0, s);
 }
 
 size_t pbs_blocksparse_matmul_back_workspace_bytes(int64_t tokens, int out_features, int in_features, int nnz,

@@ -32,6 +32,11 @@ _PROTOTYPES = {
     "pbs_blocksparse_matmul_plan_bytes": (ctypes.c_size_t, [_i32, _i32]),
     "pbs_blocksparse_matmul_plan": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp, ctypes.c_size_t, _vp]),
     "pbs_blocksparse_matmul": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _vp]),
+    "pbs_blocksparse_matmul_workspace_bytes": (ctypes.c_size_t, [_i64, _i32, _i32, _i32, _i32, _i32]),
+    "pbs_blocksparse_matmul_ws": (
+        _i32,
+        [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _vp, ctypes.c_size_t, _vp],
+    ),
     "pbs_blocksparse_matmul_back_workspace_bytes": (ctypes.c_size_t, [_i64, _i32, _i32, _i32, _i32]),
     "pbs_blocksparse_matmul_back": (
         _i32,
@@ -154,12 +159,16 @@ def blocksparse_matmul(dense_a, data, plan, n, k, nnz, transpose, bias=None, out
     tokens = dense_a.shape[0]
     if out is None:
         out = torch.empty((tokens, n), dtype=dense_a.dtype, device=dense_a.device)
+    tr, code_dtype = 1 if transpose else 0, DTYPE_CODES[dense_a.dtype]
+    # the transposed copy of the blocks that the forward bf16 kernel for dense patterns works from (made by the library)
+    ws_bytes = lib.pbs_blocksparse_matmul_workspace_bytes(tokens, n, k, nnz, tr, code_dtype)
+    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dense_a.device) if ws_bytes else None
     with torch.cuda.device(dense_a.device):
-        code = lib.pbs_blocksparse_matmul(
-            _ptr(dense_a), _ptr(data), _ptr(plan), _ptr(bias), _ptr(out), tokens, n, k, nnz,
-            1 if transpose else 0, DTYPE_CODES[dense_a.dtype], _stream(),
+        code = lib.pbs_blocksparse_matmul_ws(
+            _ptr(dense_a), _ptr(data), _ptr(plan), _ptr(bias), _ptr(out), tokens, n, k, nnz, tr, code_dtype,
+            _ptr(ws), ws_bytes, _stream(),
         )
-    _check(code, "pbs_blocksparse_matmul")
+    _check(code, "pbs_blocksparse_matmul_ws")
     return out
 
 

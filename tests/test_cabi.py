@@ -63,6 +63,25 @@ def test_matmul_argument_checks(lib):
     assert f(ctypes.c_void_p(0x1004), p, p, null, p, 4, 64, 64, 1, 1, 1, null) == ERR_ALIGN
 
 
+def test_matmul_workspace_entry_point(lib):
+    p = ctypes.c_void_p(0x1000)
+    null = ctypes.c_void_p(0)
+    f = lib.pbs_blocksparse_matmul_ws
+    assert f(p, p, p, null, p, 4, 64, 64, 1, 1, 7, null, 0, null) == ERR_DTYPE
+    assert f(p, p, p, null, p, 4, 65, 64, 1, 1, 0, null, 0, null) == ERR_SHAPE
+    assert f(p, p, p, null, p, 0, 64, 64, 1, 1, 1, null, 0, null) == OK
+    assert f(p, p, null, null, p, 4, 64, 64, 1, 1, 1, p, 1 << 20, null) == ERR_NULL
+    ws = lib.pbs_blocksparse_matmul_workspace_bytes
+    # the transposed copy of the blocks, 2 KB each: bf16, forward direction, large and dense enough
+    assert ws(16384, 4096, 4096, 8192, 1, 1) == 8192 * 2048
+    assert ws(16384, 4096, 4096, 8192, 0, 1) == 0      # the input gradient reads the data as stored
+    assert ws(16384, 4096, 4096, 8192, 1, 0) == 0      # fp32
+    assert ws(16384, 4096, 4096, 400, 1, 1) == 0       # 3 blocks per column
+    assert ws(256, 4096, 4096, 8192, 1, 1) == 0        # too few tiles
+    assert ws(16384, 4096, 8192, 16384, 1, 1) == 0     # contraction too long for the kernel's lists
+    assert ws(16384, 4096, 4096, 0, 1, 1) == 0 and ws(0, 4096, 4096, 8192, 1, 1) == 0
+
+
 def test_plan_argument_checks(lib):
     p = ctypes.c_void_p(0x1000)
     null = ctypes.c_void_p(0)
@@ -72,9 +91,15 @@ def test_plan_argument_checks(lib):
     narrow = sum(g * (128 + 2) * 16 * 4 for g in (16, 19, 22, 26))
     slots = sum((g * 8 * 4 + 63) // 64 * 64 for g in (16, 19, 22, 26))   # each table padded to 64 bytes
     wide = 8 * (64 + 2) * 64 * 4 + 256 * 4     # 8 groups of 16, 256-byte records per k-pair, progress table
-    assert nbytes == narrow + wide + slots
-    # contraction sizes that are not a multiple of 64 have no k-pair plan
+    # one column per wave: the column table of 8 groups of 16, per group a header of 64 ints, 64 k-pairs and 16 lists
+    # of up to 128 two-word items, then the table 0, 1, 2, ... of 16384 ints
+    column = 8 * 16 * 4 + (8 * (64 + 64 + 16 * 2 * 128) + 16384) * 4
+    assert nbytes == narrow + wide + slots + column
+    # contraction sizes that are not a multiple of 64 have no k-pair plans
     assert lib.pbs_blocksparse_matmul_plan_bytes(64, 96) == 4 * (1 * (3 + 2) * 16 * 4 + 64)
+    # nor does the column kernel serve contractions whose lists would not fit its LDS area
+    assert (lib.pbs_blocksparse_matmul_plan_bytes(512, 8192) - lib.pbs_blocksparse_matmul_plan_bytes(512, 8192 - 32)
+            < lib.pbs_blocksparse_matmul_plan_bytes(512, 4096) - lib.pbs_blocksparse_matmul_plan_bytes(512, 4096 - 32))
     assert lib.pbs_blocksparse_matmul_plan_bytes(100, 64) == 0
     f = lib.pbs_blocksparse_matmul_plan
     assert f(p, p, 64, 100, 1, p, 1 << 20, null) == ERR_SHAPE

@@ -1,8 +1,9 @@
-"""The wide bf16 kernel's progress protocol against its conservative variant.
+"""The progress protocol of the two barrier-free bf16 kernels against its conservative variant.
 
-In the product build a copy wave publishes "the operands of step t have landed" with one more 4-byte
+In the product build a copying wave publishes "the operands of step t have landed" with one more 4-byte
 LDS-DMA load issued behind the step's operand loads, which relies on one wave's LDS-DMA loads landing in
-issue order.  libpbs_hip_check.so is the same library compiled with -DPBS_DDS16_PUBLISH_AFTER_WAIT: there
+issue order.  libpbs_hip_check.so is the same library compiled with -DPBS_DDS16_PUBLISH_AFTER_WAIT
+-DPBS_DDSC_PUBLISH_AFTER_WAIT: there
 the copy wave waits for all its loads (s_waitcnt vmcnt(0)) and then writes the number itself, which relies
 on nothing.  If the ordering assumption failed, compute waves of the product build would multiply operands
 that had not arrived yet and the two libraries would disagree; they must agree bit for bit.
@@ -29,8 +30,11 @@ def _binding(path):
     return mod.PbsHip(path)
 
 
+@pytest.mark.parametrize("kernel", ["wide", "column"])
 @pytest.mark.parametrize("case", ["c4", "ragged"])
-def test_product_and_conservative_protocol_agree_bitwise(cuda, case):
+def test_product_and_conservative_protocol_agree_bitwise(cuda, monkeypatch, case, kernel):
+    # which of the two kernels serves the calls below (both libraries read the variable at every call)
+    monkeypatch.setenv("PBS_COLUMN_KERNEL", "1" if kernel == "column" else "0")
     assert os.path.exists(CHECK_LIB), "libpbs_hip_check.so is not built (python -m pytorch_block_sparse_amd.csrc.build)"
     if case == "c4":
         w = workloads.WORKLOADS["c4_4096x4096_d0.25_bf16"]
@@ -39,12 +43,12 @@ def test_product_and_conservative_protocol_agree_bitwise(cuda, case):
         with torch.no_grad():
             m.data.copy_(data)
         m = m.to(cuda)
-    else:   # token tail, a last column group with one column, several tiles per workgroup
+    else:   # token tail, a last column group with two columns, several tiles per workgroup, both contractions k-pairs
         np.random.seed(5)
         torch.manual_seed(5)
-        m = BlockSparseMatrix.randn((1056, 512), 33 * 16 // 3, device=cuda, dtype=torch.bfloat16)
+        m = BlockSparseMatrix.randn((1088, 512), 34 * 16 // 3, device=cuda, dtype=torch.bfloat16)
         x = torch.randn(33000 + 7, 512).to(torch.bfloat16)
-        dy = torch.randn(33000 + 7, 1056).to(torch.bfloat16)
+        dy = torch.randn(33000 + 7, 1088).to(torch.bfloat16)
     xd, dyd = x.to(cuda), dy.to(cuda)
     product, check = _binding(native.LIB_PATH), _binding(CHECK_LIB)
     out_f, in_f = m.shape
