@@ -43,12 +43,12 @@ def test_product_and_conservative_protocol_agree_bitwise(cuda, monkeypatch, case
         with torch.no_grad():
             m.data.copy_(data)
         m = m.to(cuda)
-    else:   # token tail, a last column group with two columns, several tiles per workgroup, both contractions k-pairs
+    else:   # token tail, a last column group with four columns, several tiles per workgroup, both contractions a multiple of 128
         np.random.seed(5)
         torch.manual_seed(5)
-        m = BlockSparseMatrix.randn((1088, 512), 34 * 16 // 3, device=cuda, dtype=torch.bfloat16)
+        m = BlockSparseMatrix.randn((1152, 512), 36 * 16 // 3, device=cuda, dtype=torch.bfloat16)
         x = torch.randn(33000 + 7, 512).to(torch.bfloat16)
-        dy = torch.randn(33000 + 7, 1088).to(torch.bfloat16)
+        dy = torch.randn(33000 + 7, 1152).to(torch.bfloat16)
     xd, dyd = x.to(cuda), dy.to(cuda)
     product, check = _binding(native.LIB_PATH), _binding(CHECK_LIB)
     out_f, in_f = m.shape
