@@ -10,8 +10,8 @@ Prints ONE JSON line: effective TFLOP/s (2*M*nnz*1024 per GEMM, 3 GEMMs per step
   dense_hipblaslt  the same three GEMMs dense through torch.matmul (hipBLASLt) at the same shape,
   cpu_baseline   the CPU dense-equivalent path (oracle) timed on the host cores, full size,
   other_configs  the other benchmark configurations (1024->256 forward, the two RoBERTa feed-forward
-                 shapes in fp32, the 4096 x 4096 layer in fp32, the RoBERTa-base training step), each with its own
-                 dense comparison.
+                 shapes in fp32, the 4096 x 4096 layer in fp32 and at density 0.5 in both dtypes, the RoBERTa-base
+                 training step), each with its own dense comparison.
 
 Timing: after a settling phase and `--warmup` untimed steps, exactly `--steps` steps are timed between two
 synchronisations; an event is recorded after every kernel of every timed step.  `ms_per_step` and `value`
@@ -36,7 +36,9 @@ HBM_TBPS = 8.0
 BASELINE_WORKLOAD = "c4_4096x4096_d0.25_bf16"
 BASELINE_METRIC = "effective TFLOP/s fwd+bwd at 4096² d=0.25; % of MFMA peak; vs dense GEMM"   # as in BASELINE.json
 OTHER_LAYER_WORKLOADS = ("c1_1024x256_d0.1_fp32", "c2_768x3072_d0.5_fp32", "c3_3072x768_d0.25_zipf_fp32",
-                         "c4_4096x4096_d0.25_fp32")   # the last: the headline shape in the reference's own dtype
+                         "c4_4096x4096_d0.25_fp32",   # the headline shape in the reference's own dtype
+                         # and at the upper end of the density range the speed-up over dense is asked for
+                         "c4_4096x4096_d0.5_bf16", "c4_4096x4096_d0.5_fp32")
 ROBERTA_WORKLOAD = "c5_roberta_base_mlm_fp32"
 
 
@@ -312,13 +314,13 @@ def roberta_line(args):
 
 
 def kernel_label(w, tokens, which):
-    dname = "bf16" if w.dtype.itemsize == 2 else "f32"
+    """The kernel(s) the library runs for this GEMM, as the library itself reports them."""
+    from pytorch_block_sparse_amd import native
+
     if which == "dw":
-        return ("sdd_bf16_kernel" if dname == "bf16" else "sdd_kernel") + " (+ sdd_reduce_kernel)"
-    n, k, trans = (w.out_features, w.in_features, 0) if which == "fwd" else (w.in_features, w.out_features, 1)
-    # the library picks the wide-tile kernel for bf16 when there are at least 256 tiles of 128 tokens x 512 columns
-    wide = dname == "bf16" and k % 64 == 0 and ((tokens + 127) // 128) * ((n // 32 + 15) // 16) >= 256
-    return ("dds16_kernel" if wide else "dds_kernel") + f"<TRANS={trans}>"
+        return native.matmul_back_kernel_name(tokens, w.out_features, w.in_features, w.nnz, w.dtype)
+    n, k, transpose = (w.out_features, w.in_features, True) if which == "fwd" else (w.in_features, w.out_features, False)
+    return native.matmul_kernel_name(tokens, n, k, w.nnz, transpose, w.dtype) + ("<forward>" if transpose else "<input gradient>")
 
 
 def main():
@@ -412,9 +414,11 @@ def main():
                 "ms_per_step": o["ms_per_step"],
                 "value": o["value"],
                 "unit": "TFLOP/s",
-                "frac": o["flops_gemm"] / (o["kernel_ms"][slow] * 1e-3) / 1e12 / peak,   # slowest kernel against the fp32 peak
+                "frac": o["flops_gemm"] / (o["kernel_ms"][slow] * 1e-3) / 1e12 / peak,   # slowest kernel against the matrix peak of its dtype
                 "pct_of_mfma_peak": 100.0 * o["value"] / peak,
                 "kernel_ms": o["kernel_ms"],
+                "kernels": {k: kernel_label(ow, ow.tokens, k) for k in o["kernel_ms"]},
+                "dense_ms_per_step": o["dense"]["ms_per_step"] if "dense" in o else None,
                 "vs_dense": o["dense"]["speedup_sparse_vs_dense"] if "dense" in o else None,
             }
         try:

@@ -3,8 +3,9 @@
  *
  * Plain C: raw device pointers, sizes and a hipStream_t passed as void*.  No torch
  * types.  All pointers are caller-owned device memory; the library keeps nothing
- * after a call returns and holds no mutable global device state, so calls on
- * different streams or from different host threads do not interfere.
+ * after a call returns, so calls on different streams or from different host threads
+ * do not interfere.  Its only device state of its own: the scratch array of the entry
+ * point that allocates nothing (see there) and one diagnostic counter.
  *
  * Every entry point returns an int: 0 on success, a positive hipError_t when the HIP
  * runtime reported an error, a negative PBS_ERR_* when an argument was rejected
@@ -172,14 +173,38 @@ int pbs_blocksparse_matmul_back(const void* dense_a, const void* dense_b,
  *     is written by the product kernel of the same call first.
  *   - All calls on one GPU share that GPU's array, whatever their stream: two calls that overlap on
  *     one GPU race.  Order them on one stream, or use the workspace entry point for concurrent work.
+ *   - The first call on a GPU looks up that GPU's address of the array (hipGetSymbolAddress).  A caller that is
+ *     going to capture the call into a HIP graph calls pbs_blocksparse_matmul_back_noalloc_init() once per GPU,
+ *     with that GPU current, before the capture begins; it does the lookup and nothing else.
  */
 #define PBS_NOALLOC_SCRATCH_BYTES (64u << 20)
 size_t pbs_blocksparse_matmul_back_noalloc_max_bytes(void);
+int pbs_blocksparse_matmul_back_noalloc_init(void);
 int pbs_blocksparse_matmul_back_noalloc(const void* dense_a, const void* dense_b,
                                         const int32_t* row_start_ends_a, const int32_t* cols_a,
                                         void* data_out,
                                         int64_t tokens, int out_features, int in_features, int nnz,
                                         int dtype, void* stream);
+
+/*
+ * Diagnostics.  Neither has a counterpart in the reference.
+ *
+ * pbs_protocol_failures: the bf16 kernels for large problems (dds16_kernel, ddsc_kernel) synchronise their waves
+ * through progress words in LDS with bounded waits instead of barriers.  A wait that runs into its bound means a
+ * broken protocol; the kernel then writes NaN into the results it could not vouch for and counts the event in a
+ * device word.  This call copies the current GPU's count (since the library was loaded) to *count; it synchronises
+ * the device.  The Python layer checks it after every product when PBS_DEBUG is set and raises.
+ *
+ * pbs_blocksparse_matmul_kernel_name / ..._back_kernel_name: which kernel(s) a call with these sizes runs
+ * ("dds_kernel", "dds16_kernel", "ddsc_kernel"; "sdd_seg_kernel", "sdd_kernel", "sdd_bf16_kernel", with
+ * " + sdd_reduce_kernel" when the token range is split), for benchmark labels.  "" for arguments the product
+ * entry points reject.
+ */
+int pbs_protocol_failures(unsigned* count);
+const char* pbs_blocksparse_matmul_kernel_name(int64_t tokens, int n, int k, int nnz, int transpose, int dtype,
+                                               int with_workspace);
+const char* pbs_blocksparse_matmul_back_kernel_name(int64_t tokens, int out_features, int in_features, int nnz,
+                                                    int dtype);
 
 #ifdef __cplusplus
 }

@@ -347,6 +347,25 @@ class BlockSparseMatrixBase(torch.nn.Module):
                 "blocks holds a block position outside the %d x %d grid" % (X, Y),
                 (b2.min() < 0) | (b2[:, 0].max() >= Y) | (b2[:, 1].max() >= X),
             ))
+            # Within one list the coordinates must increase strictly (sorted, no duplicates): the weight-gradient
+            # kernels binary-search a row's entries and size their tables for at most one entry per position.
+            # And the two compressed lists and `blocks` must describe the same (row, column) for every data block.
+            where = {}
+            pos = torch.arange(nnz, device=blocks.device)
+            for name, ids, ends_name, ends, n_lists, _ in lists:
+                e = ends.long().to(blocks.device).clamp(0, nnz)
+                owner = torch.searchsorted(e[1:].contiguous(), pos, right=True)   # the list each entry belongs to
+                c, b = ids[:, 0].long().to(blocks.device), ids[:, 1].long().to(blocks.device)
+                same = owner[1:] == owner[:-1]
+                problems.append(("the coordinates of %s should increase strictly within each of its lists" % name,
+                                 (same & (c[1:] <= c[:-1])).any()))
+                at = torch.full((nnz, 2), -1, dtype=torch.long, device=blocks.device)
+                at[b.clamp(0, nnz - 1)] = torch.stack((owner, c), 1)
+                where[name] = at
+            rc_a = where["cols_a"]                 # (row, column) of every data block according to the row lists
+            rc_b = where["rows_b"].flip(1)         # the column lists hold (column, row)
+            problems.append(("cols_a and rows_b should hold the same blocks", (rc_a != rc_b).any()))
+            problems.append(("blocks should hold the (column, row) of every data block of cols_a", (b2 != rc_a.flip(1)).any()))
         flags = torch.stack([p[1].to(self.blocks.device) for p in problems]).tolist()
         for (message, _), broken in zip(problems, flags):
             if broken:
@@ -354,12 +373,21 @@ class BlockSparseMatrixBase(torch.nn.Module):
 
     def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
         """Index buffers copied in from a checkpoint are validated before any kernel reads them."""
+        names = ("blocks", "cols_a", "row_start_ends_a", "rows_b", "col_start_ends_b")
+        before = {n: getattr(self, n).clone() for n in names}
         super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
         error_msgs = args[4] if len(args) > 4 else kwargs.get("error_msgs")
         self._plans = {}
         try:
             self.validate_indices()
         except Exception as e:  # reported the way torch reports the other problems of a state dict
+            # a caller that catches the error must not be left with index buffers no kernel may read
+            for n in names:
+                cur = getattr(self, n)
+                if cur.shape == before[n].shape:
+                    cur.copy_(before[n])
+                else:
+                    setattr(self, n, before[n])
             if error_msgs is None:
                 raise
             error_msgs.append("%sindex buffers are inconsistent: %s" % (prefix, e))

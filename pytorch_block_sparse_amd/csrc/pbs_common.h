@@ -102,6 +102,13 @@ typedef int __attribute__((address_space(3))) lds_int;
 static __device__ __forceinline__ int lds_peek(const int* p) { return *(const volatile lds_int*)p; }
 static __device__ __forceinline__ void lds_poke(int* p, int v) { *(volatile lds_int*)p = v; }
 
+// Waits of the barrier-free kernels that ran into their bound, counted over the life of the process (one word per
+// GPU).  Such a wait means a broken progress protocol; the kernel also turns the affected results into NaN.
+static __device__ unsigned g_protocol_failures;
+static __device__ __forceinline__ void count_protocol_failure() {
+    if ((threadIdx.x & 63) == 0) atomicAdd(&g_protocol_failures, 1u);
+}
+
 // a wave-uniform pointer, forced into scalar registers
 static __device__ __forceinline__ const unsigned char* uniform_ptr(const unsigned char* p) {
     const uint64_t v = reinterpret_cast<uint64_t>(p);

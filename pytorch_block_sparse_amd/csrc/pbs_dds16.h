@@ -325,7 +325,10 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
                 __builtin_amdgcn_s_sleep(D16_SLEEP);
             }
             // Cannot happen unless the protocol is broken: say so; the compute waves mark their results.
-            if (!free_now) lds_poke(s_fail, 1);
+            if (!free_now) {
+                lds_poke(s_fail, 1);
+                count_protocol_failure();
+            }
             wait_dma(63 - C::MAX_STEP_DMA - 1);   // the counter of outstanding loads has 6 bits
             asm volatile("" ::: "memory");
             const int n_t = issue_step(stage, vrec, e0, cnt);
@@ -493,7 +496,10 @@ __global__ __launch_bounds__((8 + NP) * 64) void dds16_kernel(D16Args g) {
                 }
                 // Operands that never arrive mean a broken protocol, not a slow machine (a wave that is
                 // not running does not count polls).  Make the failure visible: the tiles become NaN.
-                if (landed <= u) gave_up = true;
+                if (landed <= u) {
+                    gave_up = true;
+                    count_protocol_failure();
+                }
             }
             asm volatile("" ::: "memory");   // operand reads stay behind the poll
             const unsigned mask = (unsigned)__builtin_amdgcn_readlane(vrec, D16_F_MASK);

@@ -497,6 +497,7 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
         if (!here) {
             gave_up = true;
             if (lane == 0) lds_poke(s_fail, 1);
+            count_protocol_failure();
         }
     };
     // after the last item: copy this wave's remaining steps

@@ -699,6 +699,11 @@ int pbs_blocksparse_matmul_back(const void* dense_a, const void* dense_b, const 
 
 size_t pbs_blocksparse_matmul_back_noalloc_max_bytes(void) { return PBS_NOALLOC_SCRATCH_BYTES; }
 
+int pbs_blocksparse_matmul_back_noalloc_init(void) {
+    void* ws = nullptr;
+    return scratch_of_current_device(&ws);
+}
+
 int pbs_blocksparse_matmul_back_noalloc(const void* dense_a, const void* dense_b, const int32_t* row_start_ends_a,
                                         const int32_t* cols_a, void* data_out, int64_t tokens, int out_features,
                                         int in_features, int nnz, int dtype, void* stream) {
@@ -711,6 +716,31 @@ int pbs_blocksparse_matmul_back_noalloc(const void* dense_a, const void* dense_b
     }
     return pbs_blocksparse_matmul_back(dense_a, dense_b, row_start_ends_a, cols_a, data_out, tokens, out_features,
                                        in_features, nnz, dtype, ws, need, stream);
+}
+
+int pbs_protocol_failures(unsigned* count) {
+    if (!count) return PBS_ERR_NULL_POINTER;
+    return (int)hipMemcpyFromSymbol(count, HIP_SYMBOL(g_protocol_failures), sizeof(unsigned), 0, hipMemcpyDeviceToHost);
+}
+
+const char* pbs_blocksparse_matmul_kernel_name(int64_t tokens, int n, int k, int nnz, int transpose, int dtype,
+                                               int with_workspace) {
+    if ((dtype != PBS_DTYPE_F32 && dtype != PBS_DTYPE_BF16) || tokens <= 0 || n <= 0 || k <= 0 || (n % 32) || (k % 32)) return "";
+    if (dtype == PBS_DTYPE_BF16) {
+        if ((!transpose || with_workspace) && column_kernel_fits(tokens, n, k, nnz, nullptr)) return "ddsc_kernel";
+        if (wide_kernel_fits(tokens, n, k)) return "dds16_kernel";
+    }
+    return "dds_kernel";
+}
+
+const char* pbs_blocksparse_matmul_back_kernel_name(int64_t tokens, int out_features, int in_features, int nnz, int dtype) {
+    if ((dtype != PBS_DTYPE_F32 && dtype != PBS_DTYPE_BF16) || tokens <= 0 || out_features <= 0 || in_features <= 0 ||
+        nnz <= 0 || (out_features % 32) || (in_features % 32))
+        return "";
+    const SddPlan p = plan_sdd_for(dtype, tokens, out_features, in_features, nnz);
+    if (dtype == PBS_DTYPE_BF16) return p.nsplit > 1 ? "sdd_bf16_kernel + sdd_reduce_kernel" : "sdd_bf16_kernel";
+    if (p.shape >= SDD_F32_SEGMENTS) return p.nsplit > 1 ? "sdd_seg_kernel + sdd_reduce_kernel" : "sdd_seg_kernel";
+    return p.nsplit > 1 ? "sdd_kernel + sdd_reduce_kernel" : "sdd_kernel";
 }
 
 }  // extern "C"

@@ -157,6 +157,7 @@ __global__ __launch_bounds__(NW * 64) void sdd_kernel(SddArgs a) {
             my_lo = l;
             while (l < hi && a.idx[2 * l] < c0 + SC) ++l;
             my_n = l - my_lo;
+            if (my_n > SC) my_n = SC;   // (a list with repeated columns: never more entries than the tables hold)
         }
         s_rowoff[tid] = my_n;
     }

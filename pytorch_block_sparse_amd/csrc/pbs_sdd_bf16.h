@@ -163,7 +163,7 @@ static __device__ __forceinline__ void sdd_bf16_prologue(const SddArgs& a, int t
                 const bool m = (b0 + lane < n) && mine_of(s_ecol[off + b0 + lane]) >= 0;
                 cnt += __popcll(__ballot(m));
             }
-            if (lane == 0) s_rowoff[r] = cnt;
+            if (lane == 0) s_rowoff[r] = cnt < SC ? cnt : SC;   // (repeated columns: never more than the tables hold)
         }
     } else {
         if (tid < SC / 2) {
@@ -182,6 +182,7 @@ static __device__ __forceinline__ void sdd_bf16_prologue(const SddArgs& a, int t
                 my_lo = l;
                 while (l < hi && a.idx[2 * l] < c0 + SC) ++l;
                 my_n = l - my_lo;
+                if (my_n > SC) my_n = SC;
             }
             s_rowoff[tid] = my_n;
         }
@@ -212,8 +213,8 @@ static __device__ __forceinline__ void sdd_bf16_prologue(const SddArgs& a, int t
             for (int b0 = 0; b0 < n; b0 += 64) {
                 const int cl = (b0 + lane < n) ? mine_of(s_ecol[off + b0 + lane]) : -1;
                 const unsigned long long bal = __ballot(cl >= 0);
-                if (cl >= 0) {
-                    const int at = run + __popcll(bal & ((1ull << lane) - 1ull));
+                const int at = run + __popcll(bal & ((1ull << lane) - 1ull));
+                if (cl >= 0 && at < s_rowoff[r + 1]) {
                     int b = s_eblk[off + b0 + lane];
                     if (b < 0 || b >= a.nnz) b = -1;
                     s_blk[at] = b;

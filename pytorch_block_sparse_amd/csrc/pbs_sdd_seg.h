@@ -188,6 +188,7 @@ __global__ __launch_bounds__(NW * 64) void sdd_seg_kernel(SddArgs a) {
                 if (c >= cw + SC || c > c_hi) break;
                 my_n += in_segment(c) ? 1 : 0;
             }
+            if (my_n > SC) my_n = SC;   // (a list with repeated columns: never more entries than the tables hold)
         }
         if (tid < SR) s_rowoff[tid] = my_n;
         __syncthreads();
@@ -208,6 +209,7 @@ __global__ __launch_bounds__(NW * 64) void sdd_seg_kernel(SddArgs a) {
                 const int c = col_of(tid, k);
                 if (c >= cw + SC || c > c_hi) break;
                 if (!in_segment(c)) continue;
+                if (o >= s_rowoff[tid] + my_n) break;
                 int b = blk_of(tid, k);
                 if (b < 0 || b >= a.nnz) b = -1;
                 s_blk[o] = b;

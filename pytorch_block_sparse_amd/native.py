@@ -43,6 +43,10 @@ _PROTOTYPES = {
         [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _vp, ctypes.c_size_t, _vp],
     ),
     "pbs_blocksparse_matmul_back_noalloc_max_bytes": (ctypes.c_size_t, []),
+    "pbs_blocksparse_matmul_back_noalloc_init": (_i32, []),
+    "pbs_protocol_failures": (_i32, [ctypes.POINTER(ctypes.c_uint)]),
+    "pbs_blocksparse_matmul_kernel_name": (ctypes.c_char_p, [_i64, _i32, _i32, _i32, _i32, _i32, _i32]),
+    "pbs_blocksparse_matmul_back_kernel_name": (ctypes.c_char_p, [_i64, _i32, _i32, _i32, _i32]),
     "pbs_blocksparse_matmul_back_noalloc": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _vp]),
 }
 
@@ -79,6 +83,36 @@ def error_string(code):
 def _check(code, what):
     if code != 0:
         raise RuntimeError(f"{what} failed with code {code}: {error_string(code)}")
+
+
+_failures_seen = {}
+
+
+def check_protocol(what):
+    """With PBS_DEBUG set: raise if a bounded wait of a barrier-free kernel has run out since the last check
+    (the kernel marks the affected results NaN and counts the event; without this the call reports success)."""
+    if not os.environ.get("PBS_DEBUG"):
+        return
+    count = ctypes.c_uint(0)
+    _check(load().pbs_protocol_failures(ctypes.byref(count)), "pbs_protocol_failures")
+    dev = torch.cuda.current_device()
+    before = _failures_seen.get(dev, 0)
+    _failures_seen[dev] = count.value
+    if count.value != before:
+        raise RuntimeError(
+            f"{what}: {count.value - before} wait(s) of the kernel's progress protocol ran into their bound; "
+            "the results of the affected tiles are NaN"
+        )
+
+
+def matmul_kernel_name(tokens, n, k, nnz, transpose, dtype, with_workspace=True):
+    """Which kernel pbs_blocksparse_matmul_ws runs for these sizes (for benchmark labels)."""
+    return load().pbs_blocksparse_matmul_kernel_name(
+        tokens, n, k, nnz, 1 if transpose else 0, DTYPE_CODES[dtype], 1 if with_workspace else 0).decode()
+
+
+def matmul_back_kernel_name(tokens, out_features, in_features, nnz, dtype):
+    return load().pbs_blocksparse_matmul_back_kernel_name(tokens, out_features, in_features, nnz, DTYPE_CODES[dtype]).decode()
 
 
 def _stream():
@@ -169,6 +203,7 @@ def blocksparse_matmul(dense_a, data, plan, n, k, nnz, transpose, bias=None, out
             _ptr(ws), ws_bytes, _stream(),
         )
     _check(code, "pbs_blocksparse_matmul_ws")
+    check_protocol("pbs_blocksparse_matmul_ws")
     return out
 
 

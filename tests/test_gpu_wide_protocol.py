@@ -67,3 +67,26 @@ def test_product_and_conservative_protocol_agree_bitwise(cuda, monkeypatch, case
         for r in results[1:]:
             assert torch.equal(r, results[0]), f"{case}: transpose={transpose}: the two protocols disagree"
         assert torch.isfinite(results[0].float()).all()
+
+
+def test_no_wait_runs_into_its_bound(cuda, monkeypatch):
+    """With PBS_DEBUG set the Python layer reads the library's count of protocol waits that ran out after every
+    product and raises if it has grown: both barrier-free kernels, both directions, on the benchmark layer."""
+    import ctypes
+
+    monkeypatch.setenv("PBS_DEBUG", "1")
+    w = workloads.WORKLOADS["c4_4096x4096_d0.25_bf16"]
+    blocks, data, x, dy = workloads.make_inputs(w, tokens=8192)
+    m = BlockSparseMatrix.zeros((w.out_features, w.in_features), blocks=blocks, device="cpu", dtype=w.dtype)
+    with torch.no_grad():
+        m.data.copy_(data)
+    m = m.to(cuda)
+    xd, dyd = x.to(cuda), dy.to(cuda)
+    for kernel in ("0", "1"):
+        monkeypatch.setenv("PBS_COLUMN_KERNEL", kernel)
+        for _ in range(3):
+            m.reverse_matmul(xd, True)     # raises if a wait ran out
+            m.reverse_matmul(dyd, False)
+    count = ctypes.c_uint(123)
+    assert native.load().pbs_protocol_failures(ctypes.byref(count)) == 0
+    assert count.value == 0

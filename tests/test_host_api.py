@@ -183,7 +183,7 @@ def test_corrupt_index_buffers_are_rejected():
     raises from load_state_dict instead of reaching a kernel."""
     np.random.seed(0)
     torch.manual_seed(0)
-    a = BlockSparseLinear(64, 128, True, density=0.5, device="cpu")
+    a = BlockSparseLinear(64, 128, True, density=0.75, device="cpu")
     good = {k: v.clone() for k, v in a.state_dict().items()}
     nnz = a.weight.cols_a.shape[0]
 
@@ -202,14 +202,35 @@ def test_corrupt_index_buffers_are_rejected():
         "data block id used twice": corrupt("rows_b", lambda t: t.__setitem__((0, 1), int(t[1, 1]))),
         "block position outside the grid": corrupt("blocks", lambda t: t.__setitem__(0, 1000)),
     }
+    # a block row of this pattern that holds two blocks: its two entries, in turn, repeated (a duplicate
+    # position), swapped (unsorted), and given each other's data blocks (the lists disagree)
+    ends = a.weight.row_start_ends_a.tolist()
+    e0 = next(ends[r] for r in range(len(ends) - 1) if ends[r + 1] - ends[r] >= 2)
+
+    def swap_coords(t):
+        t[e0, 0], t[e0 + 1, 0] = int(t[e0 + 1, 0]), int(t[e0, 0])
+
+    def swap_blocks(t):
+        t[e0, 1], t[e0 + 1, 1] = int(t[e0 + 1, 1]), int(t[e0, 1])
+
+    cases["the same block column twice in a row"] = corrupt("cols_a", lambda t: t.__setitem__((e0 + 1, 0), int(t[e0, 0])))
+    cases["a row's block columns out of order"] = corrupt("cols_a", swap_coords)
+    cases["the two lists disagree about a block"] = corrupt("cols_a", swap_blocks)
     for what, sd in cases.items():
-        b = BlockSparseLinear(64, 128, True, density=0.5, device="cpu")
+        b = BlockSparseLinear(64, 128, True, density=0.75, device="cpu")
+        mine = {k: getattr(b.weight, k).clone() for k in INDEX_NAMES}
         with pytest.raises(RuntimeError, match="index buffers are inconsistent"):
             b.load_state_dict(sd)
-        # direct use of the check on the module that now holds the bad buffers
+        # the module is left with the index buffers it had before the load, which are consistent
+        for k in INDEX_NAMES:
+            assert torch.equal(getattr(b.weight, k), mine[k]), (what, k)
+        b.weight.validate_indices()
+        # direct use of the check on bad buffers
+        for k in INDEX_NAMES:
+            getattr(b.weight, k).copy_(sd["weight." + k])
         with pytest.raises(Exception):
             b.weight.validate_indices()
-    b = BlockSparseLinear(64, 128, True, density=0.5, device="cpu")
+    b = BlockSparseLinear(64, 128, True, density=0.75, device="cpu")
     b.load_state_dict(good)   # the untouched state dict still loads
     b.weight.validate_indices()
     # sanity_check keeps the reference's signature and conditions

@@ -47,6 +47,38 @@ def _both(lib, dy, x, ptr, cols, dtype):
     return need, ref, got
 
 
+def test_no_alloc_entry_point_under_graph_capture(cuda):
+    """The caller this entry point is for: a stream under HIP graph capture.  The address of the scratch array is
+    looked up by pbs_blocksparse_matmul_back_noalloc_init() before the capture begins (this test comes first in the
+    file, so in a fresh process that lookup is the library's first); the captured call, whose partial sums go
+    through the array, is replayed several times with eager calls that use the same array in between, and every
+    replay must give the eager result of the workspace entry point."""
+    lib = native.load()
+    assert lib.pbs_blocksparse_matmul_back_noalloc_init() == 0
+    dtype = torch.bfloat16
+    dy, x, ptr, cols = _problem(1024, 1024, 4096, 0.5, dtype, 1, cuda)
+    need, ref, got = _both(lib, dy, x, ptr, cols, dtype)   # eager: also raises the kernel's LDS limit before the capture
+    assert need > 0 and torch.equal(ref, got)
+    tokens, out_f = dy.shape
+    in_f, nnz, code = x.shape[1], cols.shape[0], native.DTYPE_CODES[dtype]
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    out = torch.full((nnz * 32, 32), -3.0, dtype=dtype, device=cuda)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        rc = lib.pbs_blocksparse_matmul_back_noalloc(p(dy), p(x), p(ptr), p(cols), p(out), tokens, out_f, in_f, nnz, code, stream)
+    assert rc == 0, native.error_string(rc)
+    dy2, x2, ptr2, cols2 = _problem(512, 768, 1000, 0.3, dtype, 2, cuda)
+    for replay in range(3):
+        out.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref), f"replay {replay}"
+        _, ref2, got2 = _both(lib, dy2, x2, ptr2, cols2, dtype)   # eager work on the same scratch array in between
+        assert torch.equal(ref2, got2)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_no_alloc_entry_point_matches_workspace_entry_point(cuda, dtype):
     lib = native.load()
