@@ -115,8 +115,31 @@ def matmul_back_kernel_name(tokens, out_features, in_features, nnz, dtype):
     return load().pbs_blocksparse_matmul_back_kernel_name(tokens, out_features, in_features, nnz, DTYPE_CODES[dtype]).decode()
 
 
-def _stream():
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+def _stream(index=None):
+    """The current stream of device `index` (default: the current device) as a hipStream_t."""
+    if index is None:
+        index = torch.cuda.current_device()
+    raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)   # the handle without a Stream object around it
+    return ctypes.c_void_p(raw(index) if raw is not None else torch.cuda.current_stream(index).cuda_stream)
+
+
+class _on_device:
+    """`with torch.cuda.device(d)` only when d is not the current device already (the context manager costs
+    several microseconds, which is most of a small product's host time)."""
+
+    def __init__(self, device):
+        self.index = device.index if device.index is not None else torch.cuda.current_device()
+        self.ctx = None if self.index == torch.cuda.current_device() else torch.cuda.device(self.index)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+        return self.index
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+        return False
 
 
 def _ptr(t):
@@ -182,27 +205,34 @@ def blocksparse_matmul_plan(ptr, indices, n, k):
 
 def blocksparse_matmul(dense_a, data, plan, n, k, nnz, transpose, bias=None, out=None):
     """out[tokens, n] = dense_a[tokens, k] . W^T (transpose) or . W (not transpose)."""
-    lib = load()
-    _require_cuda(dense_a, data, plan, bias)
-    if dense_a.dtype not in DTYPE_CODES:
-        raise RuntimeError(f"unsupported dtype {dense_a.dtype}; supported: {SUPPORTED_DTYPES}")
-    if data.dtype != dense_a.dtype:
-        raise RuntimeError(f"dense operand is {dense_a.dtype} but the block data is {data.dtype}")
-    if bias is not None and bias.dtype != dense_a.dtype:
-        raise RuntimeError(f"bias is {bias.dtype}, expected {dense_a.dtype}")
+    lib = _lib or load()
+    dtype = dense_a.dtype
+    if not (dense_a.is_cuda and data.is_cuda and plan.is_cuda and (bias is None or bias.is_cuda)):
+        _require_cuda(dense_a, data, plan, bias)
+    code_dtype = DTYPE_CODES.get(dtype)
+    if code_dtype is None:
+        raise RuntimeError(f"unsupported dtype {dtype}; supported: {SUPPORTED_DTYPES}")
+    if data.dtype != dtype:
+        raise RuntimeError(f"dense operand is {dtype} but the block data is {data.dtype}")
+    if bias is not None and bias.dtype != dtype:
+        raise RuntimeError(f"bias is {bias.dtype}, expected {dtype}")
     tokens = dense_a.shape[0]
     if out is None:
-        out = torch.empty((tokens, n), dtype=dense_a.dtype, device=dense_a.device)
-    tr, code_dtype = 1 if transpose else 0, DTYPE_CODES[dense_a.dtype]
+        out = torch.empty((tokens, n), dtype=dtype, device=dense_a.device)
+    tr = 1 if transpose else 0
     # the transposed copy of the blocks that the forward bf16 kernel for dense patterns works from (made by the library)
-    ws_bytes = lib.pbs_blocksparse_matmul_workspace_bytes(tokens, n, k, nnz, tr, code_dtype)
-    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dense_a.device) if ws_bytes else None
-    with torch.cuda.device(dense_a.device):
+    ws, ws_bytes = None, 0
+    if tr and code_dtype == 1:
+        ws_bytes = lib.pbs_blocksparse_matmul_workspace_bytes(tokens, n, k, nnz, tr, code_dtype)
+        if ws_bytes:
+            ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dense_a.device)
+    with _on_device(dense_a.device) as index:
         code = lib.pbs_blocksparse_matmul_ws(
             _ptr(dense_a), _ptr(data), _ptr(plan), _ptr(bias), _ptr(out), tokens, n, k, nnz, tr, code_dtype,
-            _ptr(ws), ws_bytes, _stream(),
+            _ptr(ws), ws_bytes, _stream(index),
         )
-    _check(code, "pbs_blocksparse_matmul_ws")
+    if code != 0:
+        _check(code, "pbs_blocksparse_matmul_ws")
     check_protocol("pbs_blocksparse_matmul_ws")
     return out
 
@@ -221,10 +251,10 @@ def blocksparse_matmul_back(dense_a, dense_b, row_start_ends_a, cols_a, out):
     code_dtype = DTYPE_CODES[dense_a.dtype]
     ws_bytes = lib.pbs_blocksparse_matmul_back_workspace_bytes(tokens, out_features, in_features, nnz, code_dtype)
     ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dense_a.device) if ws_bytes else None
-    with torch.cuda.device(dense_a.device):
+    with _on_device(dense_a.device) as index:
         code = lib.pbs_blocksparse_matmul_back(
             _ptr(dense_a), _ptr(dense_b), _ptr(row_start_ends_a), _ptr(cols_a), _ptr(out), tokens, out_features,
-            in_features, nnz, code_dtype, _ptr(ws), ws_bytes, _stream(),
+            in_features, nnz, code_dtype, _ptr(ws), ws_bytes, _stream(index),
         )
     _check(code, "pbs_blocksparse_matmul_back")
     return out
