@@ -158,6 +158,33 @@ int pbs_blocksparse_matmul_back(const void* dense_a, const void* dense_b,
                                 int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * The same product with the arguments of the reference's entry point blocksparse_matmul_back_cutlass
+ * (native/block_sparse_native.cpp:18-29; launcher native/block_sparse_cutlass_kernel_back.cu:118-160, which
+ * picks one of four kernels by the two memory-order flags, :145-157), for a caller that holds what the
+ * reference's call site holds (block_sparse.py:606-652): the two dense operands with a flag each, and the
+ * `blocks` list.
+ *
+ *   a_row_major / b_row_major   1: the operand is [tokens, features] row-major (a "contiguous" torch tensor, the
+ *                               reference's pytorch_contiguous_* = true); 0: it is [features, tokens] row-major,
+ *                               i.e. its transpose is contiguous (block_sparse.py:480-494)
+ *   blocks [nnz][2]             (block column, block row) of data block b, in any order (block_sparse.py:138-141)
+ *
+ * The CSR pair is derived from `blocks` on the device (three small kernels), and an operand given in the second
+ * order is transposed on the device, both into `workspace`; then pbs_blocksparse_matmul_back runs.  All of it
+ * is launched on `stream`.  workspace: 16-byte aligned device memory of
+ * pbs_blocksparse_matmul_back_blocks_workspace_bytes() bytes (index arrays + transposed operands + the partial
+ * sums of a split token range).  A caller that already holds row_start_ends_a / cols_a and row-major operands
+ * saves those steps by calling pbs_blocksparse_matmul_back.
+ */
+size_t pbs_blocksparse_matmul_back_blocks_workspace_bytes(int64_t tokens, int out_features, int in_features, int nnz,
+                                                          int dtype, int a_row_major, int b_row_major);
+int pbs_blocksparse_matmul_back_blocks(const void* dense_a, int a_row_major, const void* dense_b, int b_row_major,
+                                       void* data_out,
+                                       int64_t tokens, int out_features, int in_features,
+                                       const int32_t* blocks, int nnz,
+                                       int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * pbs_blocksparse_matmul_back for callers that cannot allocate device memory: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
  * reference.  Same arguments, same kernels and bit-identical results as pbs_blocksparse_matmul_back,

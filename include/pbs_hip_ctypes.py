@@ -31,6 +31,8 @@ PROTOTYPES = {
     "pbs_blocksparse_matmul_ws": (_i, [_p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _i, _p, _z, _p]),
     "pbs_blocksparse_matmul_back_workspace_bytes": (_z, [_l, _i, _i, _i, _i]),
     "pbs_blocksparse_matmul_back": (_i, [_p, _p, _p, _p, _p, _l, _i, _i, _i, _i, _p, _z, _p]),
+    "pbs_blocksparse_matmul_back_blocks_workspace_bytes": (_z, [_l, _i, _i, _i, _i, _i, _i]),
+    "pbs_blocksparse_matmul_back_blocks": (_i, [_p, _i, _p, _i, _p, _l, _i, _i, _p, _i, _i, _p, _z, _p]),
 }
 
 DTYPES = {torch.float32: 0, torch.bfloat16: 1}
@@ -86,4 +88,20 @@ class PbsHip:
             self._check(self.lib.pbs_blocksparse_matmul_back(
                 grad_out.data_ptr(), inp.data_ptr(), row_start_ends_a.data_ptr(), cols_a.data_ptr(),
                 data_out.data_ptr(), tokens, out_f, in_f, nnz, dt, ws.data_ptr(), nws, self._stream()), "matmul_back")
+        return data_out
+
+    def matmul_back_blocks(self, dense_a, a_row_major, dense_b, b_row_major, blocks, data_out):
+        """The reference's own call (block_sparse.py:637-652) with its arguments: ``dense_a`` is [tokens, out] when
+        ``a_row_major`` else [out, tokens] (likewise ``dense_b`` with in_features), ``blocks`` is the module's buffer."""
+        tokens = dense_a.shape[0] if a_row_major else dense_a.shape[1]
+        out_f = dense_a.shape[1] if a_row_major else dense_a.shape[0]
+        in_f = dense_b.shape[1] if b_row_major else dense_b.shape[0]
+        nnz, dt = blocks.shape[0] // 2, DTYPES[dense_a.dtype]
+        nws = self.lib.pbs_blocksparse_matmul_back_blocks_workspace_bytes(tokens, out_f, in_f, nnz, dt, int(a_row_major),
+                                                                          int(b_row_major))
+        ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=dense_a.device)
+        with torch.cuda.device(dense_a.device):
+            self._check(self.lib.pbs_blocksparse_matmul_back_blocks(
+                dense_a.data_ptr(), int(a_row_major), dense_b.data_ptr(), int(b_row_major), data_out.data_ptr(), tokens,
+                out_f, in_f, blocks.data_ptr(), nnz, dt, ws.data_ptr(), nws, self._stream()), "matmul_back_blocks")
         return data_out

@@ -697,6 +697,91 @@ int pbs_blocksparse_matmul_back(const void* dense_a, const void* dense_b, const 
     return launch_sdd<bf16_t>(a, dtype, workspace, workspace_bytes, s);
 }
 
+// ---- the reference's own signature of the sparse-output product ----
+struct BackBlocksLayout {
+    size_t row_ptr, cols_a, owner, a_t, b_t, inner, total;   // byte offsets into the workspace; inner = the split workspace
+};
+static inline size_t round256(size_t v) { return (v + 255) / 256 * 256; }
+static BackBlocksLayout back_blocks_layout(int64_t tokens, int out_features, int in_features, int nnz, int dtype,
+                                           int a_row_major, int b_row_major) {
+    BackBlocksLayout l;
+    const size_t X = out_features / 32, Y = in_features / 32, esz = dtype == PBS_DTYPE_F32 ? 4 : 2;
+    size_t off = 0;
+    l.row_ptr = off;
+    off += round256((X + 1) * sizeof(int32_t));
+    l.cols_a = off;
+    off += round256((size_t)nnz * 2 * sizeof(int32_t));
+    l.owner = off;
+    off += round256(X * Y * sizeof(int));
+    l.a_t = off;
+    if (!a_row_major) off += round256((size_t)tokens * out_features * esz);
+    l.b_t = off;
+    if (!b_row_major) off += round256((size_t)tokens * in_features * esz);
+    l.inner = off;
+    off += round256(pbs_blocksparse_matmul_back_workspace_bytes(tokens, out_features, in_features, nnz, dtype));
+    l.total = off;
+    return l;
+}
+
+size_t pbs_blocksparse_matmul_back_blocks_workspace_bytes(int64_t tokens, int out_features, int in_features, int nnz,
+                                                          int dtype, int a_row_major, int b_row_major) {
+    if (tokens < 0 || out_features <= 0 || in_features <= 0 || nnz <= 0) return 0;
+    if ((out_features % 32) || (in_features % 32)) return 0;
+    if (dtype != PBS_DTYPE_F32 && dtype != PBS_DTYPE_BF16) return 0;
+    return back_blocks_layout(tokens, out_features, in_features, nnz, dtype, a_row_major, b_row_major).total;
+}
+
+int pbs_blocksparse_matmul_back_blocks(const void* dense_a, int a_row_major, const void* dense_b, int b_row_major,
+                                       void* data_out, int64_t tokens, int out_features, int in_features,
+                                       const int32_t* blocks, int nnz, int dtype, void* workspace, size_t workspace_bytes,
+                                       void* stream) {
+    if (dtype != PBS_DTYPE_F32 && dtype != PBS_DTYPE_BF16) return PBS_ERR_BAD_DTYPE;
+    if (tokens < 0 || out_features <= 0 || in_features <= 0 || nnz < 0 || (out_features % 32) || (in_features % 32))
+        return PBS_ERR_BAD_SHAPE;
+    if (tokens > (1ll << 30) || (long long)nnz > (long long)(out_features / 32) * (in_features / 32))
+        return PBS_ERR_TOO_LARGE;
+    if (nnz == 0) return PBS_OK;
+    if (!blocks || !data_out) return PBS_ERR_NULL_POINTER;
+    if (tokens > 0 && (!dense_a || !dense_b)) return PBS_ERR_NULL_POINTER;
+    if (!aligned16(dense_a) || !aligned16(dense_b) || !aligned16(data_out)) return PBS_ERR_MISALIGNED;
+    const BackBlocksLayout l = back_blocks_layout(tokens, out_features, in_features, nnz, dtype, a_row_major, b_row_major);
+    if (!workspace || workspace_bytes < l.total || !aligned16(workspace)) return PBS_ERR_WORKSPACE;
+    unsigned char* ws = static_cast<unsigned char*>(workspace);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int X = out_features / 32, Y = in_features / 32;
+    int32_t* row_ptr = reinterpret_cast<int32_t*>(ws + l.row_ptr);
+    int32_t* cols_a = reinterpret_cast<int32_t*>(ws + l.cols_a);
+    int* owner = reinterpret_cast<int*>(ws + l.owner);
+    const long long positions = (long long)X * Y;
+    hipLaunchKernelGGL(blocks_owner_clear_kernel, dim3((unsigned)((positions + 255) / 256)), dim3(256), 0, s, owner, positions);
+    hipLaunchKernelGGL(blocks_owner_kernel, dim3((unsigned)((nnz + 255) / 256)), dim3(256), 0, s, blocks, nnz, X, Y, owner);
+    hipLaunchKernelGGL(csr_from_owner_kernel, dim3(1), dim3(INDEX_THREADS), 0, s, owner, X, Y, cols_a, row_ptr);
+    if (int rc = (int)hipGetLastError()) return rc;
+    // an operand given with the tokens along its rows' direction ([features, tokens]) is brought to [tokens, features]
+    auto to_row_major = [&](const void* src, size_t off, int features) -> int {
+        const dim3 grid((unsigned)((tokens + 31) / 32), (unsigned)((features + 31) / 32));
+        if (dtype == PBS_DTYPE_F32)
+            hipLaunchKernelGGL(transpose_dense_kernel<uint32_t>, grid, dim3(256), 0, s, static_cast<const uint32_t*>(src),
+                               reinterpret_cast<uint32_t*>(ws + off), (long long)features, (long long)tokens);
+        else
+            hipLaunchKernelGGL(transpose_dense_kernel<uint16_t>, grid, dim3(256), 0, s, static_cast<const uint16_t*>(src),
+                               reinterpret_cast<uint16_t*>(ws + off), (long long)features, (long long)tokens);
+        return (int)hipGetLastError();
+    };
+    const void* a = dense_a;
+    const void* b = dense_b;
+    if (!a_row_major && tokens > 0) {
+        if (int rc = to_row_major(dense_a, l.a_t, out_features)) return rc;
+        a = ws + l.a_t;
+    }
+    if (!b_row_major && tokens > 0) {
+        if (int rc = to_row_major(dense_b, l.b_t, in_features)) return rc;
+        b = ws + l.b_t;
+    }
+    return pbs_blocksparse_matmul_back(a, b, row_ptr, cols_a, data_out, tokens, out_features, in_features, nnz, dtype,
+                                       ws + l.inner, l.total - l.inner, stream);
+}
+
 size_t pbs_blocksparse_matmul_back_noalloc_max_bytes(void) { return PBS_NOALLOC_SCRATCH_BYTES; }
 
 int pbs_blocksparse_matmul_back_noalloc_init(void) {

@@ -115,4 +115,65 @@ __global__ __launch_bounds__(INDEX_THREADS) void build_indices_kernel(
     }
 }
 
+// ---- the CSR pair of a pattern given as the reference's `blocks` list ----
+// blocks[2 b] = block column, blocks[2 b + 1] = block row of data block b, in any order.  owner[p] = data block
+// at row-major position p of the X x Y grid, or -1; then one row-major sweep of owner writes cols_a (sorted by
+// row, then column) and the row starts.  A position listed twice keeps one of its data blocks (the other gets no
+// result); entries outside the grid are skipped.
+__global__ __launch_bounds__(256) void blocks_owner_clear_kernel(int* owner, long long total) {
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i < total) owner[i] = -1;
+}
+__global__ __launch_bounds__(256) void blocks_owner_kernel(const int32_t* __restrict__ blocks, int nnz, int X, int Y, int* owner) {
+    const int b = blockIdx.x * 256 + threadIdx.x;
+    if (b >= nnz) return;
+    const int c = blocks[2 * b], r = blocks[2 * b + 1];
+    if (c >= 0 && c < Y && r >= 0 && r < X) owner[(long long)r * Y + c] = b;
+}
+__global__ __launch_bounds__(INDEX_THREADS) void csr_from_owner_kernel(const int* __restrict__ owner, int X, int Y,
+                                                                       int32_t* cols_a, int32_t* row_ptr) {
+    __shared__ int s_wave[17];
+    const int tid = threadIdx.x;
+    const long long total = (long long)X * Y;
+    const long long chunk = (total + INDEX_THREADS - 1) / INDEX_THREADS;
+    long long lo = tid * chunk, hi = lo + chunk;
+    if (lo > total) lo = total;
+    if (hi > total) hi = total;
+    int cnt = 0;
+    for (long long p = lo; p < hi; ++p) cnt += owner[p] >= 0 ? 1 : 0;
+    int counted;
+    int rank = block_exclusive_scan(cnt, s_wave, &counted);
+    for (long long p = lo; p < hi; ++p) {
+        const int r = (int)(p / Y), c = (int)(p % Y);
+        if (c == 0) row_ptr[r] = rank;
+        const int b = owner[p];
+        if (b >= 0) {
+            cols_a[2 * rank] = c;
+            cols_a[2 * rank + 1] = b;
+            ++rank;
+        }
+    }
+    if (tid == 0) row_ptr[X] = counted;
+}
+
+// out[c][r] = in[r][c] for a rows x cols matrix of 2- or 4-byte elements (tiles of 32 x 32 through LDS)
+template <typename U>
+__global__ __launch_bounds__(256) void transpose_dense_kernel(const U* __restrict__ in, U* __restrict__ out, long long rows,
+                                                              long long cols) {
+    __shared__ U s[32][33];
+    const long long r0 = (long long)blockIdx.y * 32, c0 = (long long)blockIdx.x * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;   // 32 x 8
+#pragma unroll
+    for (int i = 0; i < 32; i += 8) {
+        const long long r = r0 + ty + i, c = c0 + tx;
+        if (r < rows && c < cols) s[ty + i][tx] = in[r * cols + c];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 32; i += 8) {
+        const long long c = c0 + ty + i, r = r0 + tx;
+        if (r < rows && c < cols) out[c * rows + r] = s[tx][ty + i];
+    }
+}
+
 }  // namespace pbs

@@ -42,6 +42,11 @@ _PROTOTYPES = {
         _i32,
         [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _vp, ctypes.c_size_t, _vp],
     ),
+    "pbs_blocksparse_matmul_back_blocks_workspace_bytes": (ctypes.c_size_t, [_i64, _i32, _i32, _i32, _i32, _i32, _i32]),
+    "pbs_blocksparse_matmul_back_blocks": (
+        _i32,
+        [_vp, _i32, _vp, _i32, _vp, _i64, _i32, _i32, _vp, _i32, _i32, _vp, ctypes.c_size_t, _vp],
+    ),
     "pbs_blocksparse_matmul_back_noalloc_max_bytes": (ctypes.c_size_t, []),
     "pbs_blocksparse_matmul_back_noalloc_init": (_i32, []),
     "pbs_protocol_failures": (_i32, [ctypes.POINTER(ctypes.c_uint)]),

@@ -26,28 +26,53 @@ class MagnitudeSparseOptimizerStrategy(SparseOptimizerStrategy):
         self.new_coefficients_scale = new_coefficients_scale
 
     def initialize_new_blocks(self, old_data, new_data):
+        # mean and std stay 0-d tensors on the data's device: nothing here waits for the GPU
         mean, std = old_data.float().mean(), old_data.float().std()
         scale = self.new_coefficients_scale
         if self.new_coefficients_distribution == "gaussian":
-            new_data.normal_(mean=float(mean * scale), std=float(std * scale))
+            new_data.normal_(mean=0.0, std=1.0)
+            new_data.mul_((std * scale).to(new_data.dtype)).add_((mean * scale).to(new_data.dtype))
         elif self.new_coefficients_distribution == "uniform":
             # The reference draws with random_(0, 1), whose only possible value is 0, so its
             # "uniform" blocks are the constant -std*scale (sparse_optimizer.py:31-34).  Kept as is.
             new_data.random_(0, 1)
             new_data -= 0.5
-            new_data *= float(2 * std * scale)
+            new_data *= (2 * std * scale).to(new_data.dtype)
         else:
             raise Exception("Unknown new coefficients method %s" % self.new_coefficients_distribution)
 
+    def free_positions(self, bsm, count):
+        """`count` distinct empty block positions chosen uniformly at random, as [count, 2] (block row, block column).
+
+        On a GPU the choice is made on the GPU: every position draws a uniform key, occupied positions get a key
+        above all others, and the `count` smallest keys win (a uniform random subset in random order, like the first
+        `count` entries of a random permutation of the empty positions, reference sparse_optimizer.py:55-56).  The
+        number of empty positions follows from the shapes, so nothing is read back.  On the CPU the reference's own
+        sequence is kept (torch.randperm over the list of empty positions), so seeded host runs choose as it does.
+        """
+        mask = bsm.block_mask_build(None)
+        X, Y = mask.shape
+        n_free = X * Y - bsm.data.shape[0] // bsm.block_shape[0]
+        if not mask.is_cuda:
+            free = (~mask).nonzero()
+            return free[torch.randperm(free.shape[0])[:count]]
+        take = min(count, n_free)
+        keys = torch.rand(X * Y, device=mask.device)
+        keys.masked_fill_(mask.view(-1), 2.0)
+        pick = torch.topk(keys, take, largest=False, sorted=True).indices
+        return torch.stack([pick // Y, pick % Y], 1)
+
     def run(self, block_sparse_matrix):
+        """reference: sparse_optimizer.py:38-87.  On a GPU every step runs there: block norms, their order, the choice
+        of empty positions, the new index buffers (block_replace -> pbs_build_indices) and the new values; the only
+        waits are the error checks of rebuild (one status word and one validation flag vector read back)."""
         bsm = block_sparse_matrix
         bs0, bs1 = bsm.block_shape
         order = bsm.block_norm().sort()[1]
         dropped = order[: int(order.shape[0] * self.cleanup_ratio)]
 
-        free = (~bsm.block_mask_build(None)).nonzero()
-        pick = torch.randperm(free.shape[0])[: dropped.shape[0]].to(free.device)
-        bsm.block_replace(torch.cat([free[pick], dropped.unsqueeze(-1)], -1))
+        positions = self.free_positions(bsm, dropped.shape[0])
+        bsm.block_replace(torch.cat([positions, dropped.unsqueeze(-1)], -1))
 
         fresh = torch.zeros(bsm.data.shape[0] // bs0, dtype=torch.bool, device=bsm.data.device)
         fresh[dropped] = True

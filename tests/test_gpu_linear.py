@@ -189,6 +189,52 @@ def test_patched_model_trains_and_sparse_optimizer(cuda, capsys):
     assert all(np.isfinite(losses)) and losses[-1] < losses[0]
 
 
+def test_magnitude_strategy_on_the_device(cuda):
+    """MagnitudeSparseOptimizerStrategy.run with the matrix on the GPU (reference sparse_optimizer.py:38-87): the
+    blocks it drops are exactly the lowest-norm ones, the positions it fills were empty and are distinct, the blocks it
+    keeps stay where they were with their values, the regrown blocks get the new values, and the choice of
+    positions is random under the device generator's seed."""
+    from pytorch_block_sparse_amd.sparse_optimizer import MagnitudeSparseOptimizerStrategy
+
+    def one(seed, distribution):
+        np.random.seed(11)
+        torch.manual_seed(11)
+        m = BlockSparseMatrix.randn((512, 384), 70, device=cuda)
+        with torch.no_grad():   # distinct block norms
+            m.data.mul_(torch.linspace(0.5, 2.0, 70, device=cuda).repeat_interleave(32).unsqueeze(1))
+        norms = m.block_norm().clone()
+        pos0 = m.build_coo_block_index().t().clone()    # (row, column) by data block
+        data0 = m.data.detach().clone()
+        mask0 = m.block_mask_build(None).clone()
+        torch.manual_seed(seed)
+        keep = MagnitudeSparseOptimizerStrategy(0.2, distribution, 0.1).run(m)
+        return m, norms, pos0, data0, mask0, keep
+
+    m, norms, pos0, data0, mask0, keep = one(1, "gaussian")
+    k = int(70 * 0.2)
+    dropped = norms.sort()[1][:k]
+    kept = norms.sort()[1][k:]
+    pos1 = m.build_coo_block_index().t()
+    assert torch.equal(pos1[kept], pos0[kept])                       # kept blocks did not move
+    new_pos = pos1[dropped]
+    assert not mask0[new_pos[:, 0], new_pos[:, 1]].any()             # regrown where nothing was
+    assert torch.unique(new_pos[:, 0] * 12 + new_pos[:, 1]).numel() == k
+    assert int(m.block_mask_build(None).sum()) == 70
+    d0, d1 = data0.view(70, -1), m.data.detach().view(70, -1)
+    assert torch.equal(d1[kept], d0[kept])                           # nor did their values change
+    fresh = d1[dropped]
+    assert abs(fresh.std().item() / (0.1 * data0.std().item()) - 1.0) < 0.05
+    assert torch.equal(keep.view(70, -1)[:, 0] == 0, torch.isin(torch.arange(70, device=cuda), dropped))
+    m.check_with_dense(m.to_dense())
+    # the reference's "uniform" is the constant -std * scale (random_(0, 1) only draws 0)
+    mu, _, _, data0u, _, _ = one(1, "uniform")
+    assert torch.allclose(mu.data.detach().view(70, -1)[dropped], (-0.1 * data0u.std()).expand(k, 1024), rtol=1e-5)
+    # same seed, same choice; another seed, another choice
+    again = one(1, "gaussian")[0].build_coo_block_index().t()[dropped]
+    other = one(2, "gaussian")[0].build_coo_block_index().t()[dropped]
+    assert torch.equal(again, new_pos) and not torch.equal(other, new_pos)
+
+
 def test_roberta_patched_at_full_density_keeps_outputs(cuda):
     """reference tests/test_integration.py:66-113 (test1), two encoder layers instead of six: patching the
     feed-forward linears of a RoBERTa masked-LM model at density 1.0 keeps parameter count and logits;

@@ -88,3 +88,45 @@ def test_reference_side_binding_against_oracle(cuda, dtype):
     # the plan belongs to the pattern: the old one gives the old pattern's product, not the new one's
     assert not torch.equal(plan_old, plan_new)
     assert not torch.allclose(y_old.float(), y_new.float())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_reference_signature_of_the_sparse_output_product(cuda, dtype):
+    """pbs_blocksparse_matmul_back_blocks takes what the reference's blocksparse_matmul_back_cutlass takes
+    (native/block_sparse_native.cpp:18-29): each dense operand in either memory order with its flag, and the `blocks`
+    list instead of the CSR pair.  All four flag combinations (the four kernels of
+    native/block_sparse_cutlass_kernel_back.cu:145-157) against the oracle, on a pattern whose data blocks are not in
+    row-major order (the state after a block_replace) and with a token count that splits the token range."""
+    binding = _binding()
+    lib = binding.PbsHip(LIB)
+    out_f, in_f, tokens = 384, 320, 4099
+    X, Y = out_f // 32, in_f // 32
+    rng = np.random.RandomState(3)
+    mask = rng.rand(X, Y) < 0.35
+    mask[5, :] = False
+    nnz = int(mask.sum())
+    block_ptr = rng.permutation(nnz)            # data block of the i-th nonzero in row-major order
+    idx = O.build_indices(mask, block_ptr)
+    coo = O.build_coo_block_index(idx["row_start_ends_a"], idx["cols_a"])
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(tokens, in_f, generator=g).to(dtype)
+    dy = torch.randn(tokens, out_f, generator=g).to(dtype)
+    data = torch.zeros(nnz * 32, 32).to(dtype)
+    _, _, dw_ref = O.linear_fwd_bwd(x.double().numpy(), dy.double().numpy(), data.double().numpy(), coo, (out_f, in_f))
+    blocks = torch.from_numpy(np.ascontiguousarray(idx["blocks"])).to(cuda)
+    xd, dyd = x.to(cuda), dy.to(cuda)
+    xt, dyt = xd.t().contiguous(), dyd.t().contiguous()    # [features, tokens]: "the transpose is contiguous"
+    results = []
+    for a_rm in (True, False):
+        for b_rm in (True, False):
+            print(f"memory orders a_row_major={a_rm} b_row_major={b_rm} {dtype}", flush=True)
+            out = torch.full((nnz * 32, 32), float("nan"), dtype=dtype, device=cuda)
+            lib.matmul_back_blocks(dyd if a_rm else dyt, a_rm, xd if b_rm else xt, b_rm, blocks, out)
+            assert_close(out, dw_ref, dtype, f"a_row_major={a_rm} b_row_major={b_rm}")
+            results.append(out)
+    for r in results[1:]:
+        assert torch.equal(r, results[0])       # the memory order of an operand does not change a bit of the result
+    # and it is the result of the entry point that takes the CSR pair
+    d = _device_indices(idx, cuda)
+    ref = lib.matmul_back(dyd, xd, d["row_start_ends_a"], d["cols_a"], torch.empty_like(results[0]))
+    assert torch.equal(ref, results[0])
