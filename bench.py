@@ -127,6 +127,47 @@ def time_steps(kernels, steps, warmup):
     return median(per_step), mean_ms, per_kernel
 
 
+def forward_latency(call, n_graph=20):
+    """Latency figures of a small forward product, in microseconds per call: `host_issue` = wall time of back-to-back
+    calls without synchronisation (what the Python + ctypes path costs; the GPU keeps up), `graph_replay` = the call
+    captured n_graph times into one HIP graph and replayed (kernel time plus the gap between two launches, no host
+    path), next to the event figure of time_steps (launch latency + kernel)."""
+    import torch
+
+    for _ in range(20):
+        call()
+    torch.cuda.synchronize()
+    n = 1000
+    t0 = time.perf_counter()
+    for _ in range(n):
+        call()
+    t1 = time.perf_counter()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            call()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(n_graph):
+            keep = call()
+    for _ in range(5):
+        graph.replay()
+    torch.cuda.synchronize()
+    per = []
+    for _ in range(50):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        per.append(e0.elapsed_time(e1) / n_graph * 1e3)
+    del keep
+    return {"host_issue": (t1 - t0) / n * 1e6, "graph_replay": median(per)}
+
+
 def cpu_baseline(w, tokens):
     """The reference's CPU dense-equivalent path (to_dense + matmul, fp32): 3 warm-up + 5 timed runs, median."""
     import torch
@@ -196,6 +237,8 @@ def measure_layer(w, tokens, steps, warmup, dense=True):
         "kernel_ms": per_kernel,
         "value": len(kernels) * flops_gemm / (ms_step * 1e-3) / 1e12,
     }
+    if w.passes == "fwd":
+        res["latency_us"] = forward_latency(kernels["fwd"])
     if dense:
         wd = m.to_dense()
         dk = {"fwd": lambda: xd @ wd.t()}
@@ -394,6 +437,8 @@ def main():
     }
     if "dense" in r:
         out["dense_hipblaslt"] = r["dense"]
+    if "latency_us" in r:
+        out["latency_us"] = r["latency_us"]
 
     if args.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.uint8, device="cuda:0").fill_(1)
@@ -417,6 +462,7 @@ def main():
                 "frac": o["flops_gemm"] / (o["kernel_ms"][slow] * 1e-3) / 1e12 / peak,   # slowest kernel against the matrix peak of its dtype
                 "pct_of_mfma_peak": 100.0 * o["value"] / peak,
                 "kernel_ms": o["kernel_ms"],
+                **({"latency_us": o["latency_us"]} if "latency_us" in o else {}),
                 "kernels": {k: kernel_label(ow, ow.tokens, k) for k in o["kernel_ms"]},
                 "dense_ms_per_step": o["dense"]["ms_per_step"] if "dense" in o else None,
                 "vs_dense": o["dense"]["speedup_sparse_vs_dense"] if "dense" in o else None,
