@@ -328,3 +328,45 @@ def test_benchmark_shape_fp32_4096(cuda):
            + m.matmul_with_output_sparse_support(dyd[half:], xd[half:]).double())
     assert (dw.double() - ref).abs().max().item() < 1e-4 * ref.abs().max().item()
     assert torch.equal(m.reverse_matmul(xd[1024:1536], True), y[1024:1536])
+
+
+def test_skewed_pattern_with_thousands_of_block_columns(cuda):
+    """A result of 3500 block columns with very uneven block counts: the slot tables of all four group widths (8, 7, 6
+    and 5 columns to a group; 3500 columns in groups of 5 are 700 groups = 5600 places) must each hold every block
+    column exactly once, and the product must be right whichever width the launch takes."""
+    out_f, in_f, tokens = 3500 * 32, 96, 40
+    X, Y = out_f // 32, in_f // 32
+    rng = np.random.RandomState(2)
+    kind = rng.rand(X)
+    blocks = []
+    for r in range(X):
+        if kind[r] < 0.05:
+            blocks += [(r, c) for c in range(Y)]          # three blocks
+        elif kind[r] < 0.75:
+            blocks.append((r, int(rng.randint(Y))))       # one
+    counts = np.bincount([r for r, _ in blocks], minlength=X)
+    assert counts.max() * X > 2 * counts.sum()            # what the library calls skewed
+    m = _matrix(out_f, in_f, blocks, None, torch.float32, cuda, seed=4)
+    from pytorch_block_sparse_amd import native
+
+    plan = native.blocksparse_matmul_plan(m.row_start_ends_a, m.cols_a, out_f, in_f).cpu().numpy()
+    # the plan buffer of a contraction that is not a multiple of 64: [records, width 8][slots 8][records 7][slots 7] ...
+    off = 0
+    for width in (8, 7, 6, 5):
+        groups = (X + width - 1) // width
+        off += groups * (Y + 2) * 16          # records: header + one per k-block + sentinel, 16 ints each
+        n_slots = groups * 8
+        slots = plan[off:off + n_slots]
+        off += (n_slots * 4 + 63) // 64 * 16
+        held = np.sort(slots[slots >= 0])
+        assert np.array_equal(held, np.arange(X)), f"width {width}: the slot table loses or repeats block columns"
+    assert off * 4 == native.load().pbs_blocksparse_matmul_plan_bytes(out_f, in_f)
+    # forward and weight gradient (the input gradient of this layer contracts over 112000 features, beyond what the
+    # kernels' plan records hold in LDS)
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn((tokens, in_f), generator=g)
+    dy = torch.randn((tokens, out_f), generator=g)
+    coo = m.build_coo_block_index().cpu().numpy()
+    y_ref, _, dw_ref = O.linear_fwd_bwd(to64(x), to64(dy), to64(m.data), coo, tuple(m.shape))
+    assert_close(m.reverse_matmul(x.to(cuda), True), y_ref, torch.float32, "3500 block columns fwd")
+    assert_close(m.matmul_with_output_sparse_support(dy.to(cuda), x.to(cuda)), dw_ref, torch.float32, "3500 block columns dw")
