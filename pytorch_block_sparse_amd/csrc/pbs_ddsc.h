@@ -10,17 +10,18 @@
 // vector-memory instruction per four cycles, shared by its four waves, so every bookkeeping instruction of an
 // item is paid several times over on the path of the wave with the most items.  Hence: everything that
 // depends on the pattern only is precomputed in the item words; a wave looks at one progress word per item;
-// waves that wait sleep long; only half of the waves copy.
+// waves that wait sleep long; and only a wave that has to wait anyway copies.
 //
 // The block columns are ranked by block count and dealt to the waves so that every SIMD of every
 // workgroup gets the same number of blocks (ddsc_cols_kernel): places 0-3 of a group (one per SIMD) hold
-// its heaviest columns, places 12-15 its lightest.  The waves of the light half (places 8-15) have time to
-// spare and do all the copying; the heavy half only multiplies.
+// its heaviest columns, places 12-15 its lightest.  Adjacent block columns stay in one group, so that the
+// two halves of a 128-byte line of the result are stored at about the same time.
 //
 // Operands.
 //   dense operand   A step is a pair of adjacent k-blocks (128-byte rows).  Its 128 x 64 panel goes
-//                   global -> LDS by DMA into a ring of RS steps (16 KB each).  Step t is copied by the
-//                   wave 8 + t % 8 (16 DMA instructions); eight copies are in flight at a time.
+//                   global -> LDS by DMA into a ring of RS steps (16 KB each).  A step is copied by
+//                   whichever wave finds itself waiting for a panel while the step's ring slot is free
+//                   (16 DMA instructions); up to RS copies are in flight at a time.
 //   packed blocks   never pass through LDS.  A block is multiplied by exactly one wave per token tile, so
 //                   the wave loads its two 16-byte fragments per lane straight from global memory into
 //                   registers, DC_L items ahead, with ordinary loads (the compiler places the waits and never
@@ -35,21 +36,27 @@
 // the registers.
 //
 // Progress words in LDS (one writer each, only growing; no barriers after the prologue):
-//   landed[c]   steps copied by copier c (wave 8 + c) whose rows have arrived (the number of the last one plus
-//               one): behind its rows of step t the wave issues one single-lane 4-byte DMA that copies the
-//               number from a table 0, 1, 2, ... in global memory onto the word; a wave's loads complete in order;
+//   landed[s]   ring slot s holds step landed[s] - 1: behind the rows of step t the copying wave issues one
+//               single-lane 4-byte DMA that copies the number t + 1 from a table 0, 1, 2, ... in global memory
+//               onto the word of slot t % RS; a wave's loads complete in order;
 //   done[w]     the global step wave w still needs: it has finished reading every earlier step (every lane
-//               writes its own copy of the word, lane 0's is read).
-// Step t may overwrite ring slot t % RS once min done[] > t - RS (the copiers poll that minimum); an item of
-// step u may be read when its copier's word exceeds u.  A wave reads that word for its next item behind the
-// current item's fragment reads and looks at it when it gets there, so the round trip is off the item's path.
+//               writes its own copy of the word, lane 0's is read);
+//   next        the first step nobody has copied yet (advanced by compare-and-swap: the one word with several
+//               writers).
+// Step t may overwrite ring slot t % RS once min done[] > t - RS; an item of step u may be read when its
+// slot's word exceeds u.  A wave reads that word for its next item behind the current item's fragment reads
+// and looks at it when it gets there, so the round trip is off the item's path.  A wave whose panel is not
+// there reads all the words at once, copies every free step it manages to claim, sleeps, and looks again:
+// the waves with few items run ahead, meet steps that are not there yet and so do most of the copying, and a
+// freed ring slot is refilled within one poll interval, whatever the other waves are busy with.  (With a
+// fixed copier per step, a slot waited for that wave to finish its own item or its epilogue: 0.203 -> 0.186 ms
+// for the input gradient of the 4096 x 4096 layer at density 0.25, 0.297 -> 0.274 at 0.5.)
 // Every wait polls with s_sleep and is bounded; a wait that runs into its bound (a broken protocol, not a slow
 // machine) makes the results NaN instead of passing silently.
 //
-// The compiler does not see the DMA instructions (inline assembly), so in a copier its wait for a block
-// also covers as many older loads as DMA instructions were issued since the block was requested; the DMA
-// is therefore issued right before that wait, where it is the youngest.  The heavy half issues no DMA and
-// waits exactly.
+// The compiler does not see the DMA instructions (inline assembly), so after a wave has copied, its next
+// wait for a block also covers the DMA instructions issued since the block was requested: it waits for its
+// own copy to land.  A wave that has not copied waits exactly.
 //
 // Persistent workgroups: a workgroup keeps one group of 16 block columns and walks several token
 // tiles; steps are numbered across tiles, so the first loads of a tile overlap the previous tile's stores.
@@ -69,7 +76,7 @@
 namespace pbs {
 
 constexpr int DC_NB = 16;               // block columns per tile = waves per workgroup
-constexpr int DC_NC = 8;                // copiers: the waves DC_NB - DC_NC .. DC_NB - 1
+constexpr int DC_NC = 8;                // words reserved for landed[] (one per ring slot)
 constexpr int DC_L = 2;                 // blocks loaded ahead of the item being multiplied
 constexpr int DC_BM = 128;              // tokens per tile
 constexpr int DC_HDR = 64;
@@ -78,7 +85,7 @@ constexpr int DC_MAX_KP = 512;          // k-pairs (K <= 32768): 9 bits of an it
 constexpr int DC_ITEM_LAST = 1 << 10;
 constexpr int DC_MAX_BLOCKS = 1 << 21;  // byte offsets of blocks stay below 2^32
 constexpr int DC_ITEMS_LDS = 2048;      // items of a group kept in LDS (every pattern up to K = 4096)
-constexpr int DC_SEQ_INTS = 16384;      // the table 0, 1, 2, ...: a workgroup's steps are numbered below this
+constexpr int DC_SEQ_INTS = 16384;      // the table 0, 1, 2, ...: a workgroup's steps are numbered below this (a power of two)
 #ifndef DC_SLEEP
 #define DC_SLEEP 8
 #endif
@@ -294,9 +301,9 @@ static __device__ __forceinline__ void dma4_lane0(unsigned lds_base_uniform, con
                  : "memory");
 }
 
-template <int RS, int NCS>
+template <int RS>
 __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
-    static_assert(NCS == 1 || NCS == 2 || NCS == 4, "copiers per step");
+    static_assert(RS <= DC_NC, "one landed word per ring slot");
     using C = DdscCfg<RS>;
     using E = Elem<bf16_t>;
     constexpr int NW = C::NW, NC = DC_NC, L = DC_L;
@@ -362,37 +369,35 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
     const unsigned char* Dp = static_cast<const unsigned char*>(g.data);
     const unsigned a_row_bytes = (unsigned)g.K * 2u;
 
-    // ---------------- copy side (waves NW - NC .. NW - 1) ----------------
-    const bool copier = wave >= NW - NC;
-    const int cidx = wave - (NW - NC);
-    constexpr int G = NC / NCS;              // groups of NCS copiers; group i copies the steps t with t % G == i
-    constexpr int CROWS = C::BM / NCS;       // rows of a step one copier copies
-    const int my_phase = (cidx / NCS) & (G - 1);
-    const int my_rows = (cidx % NCS) * CROWS;
-    // Lane l of DMA instruction i of a step: row my_rows + 8 i + l / 8, physical chunk l % 8 = logical chunk
-    // (l % 8) ^ ((row / 2) % 8).  my_rows is a multiple of 32, so the swizzle term is (l / 16) for even i and
-    // (l / 16) ^ 4 for odd i: two per-lane offsets serve all rows (the row advances in the scalar base address).
-    const unsigned char* a_tile = A;
-    int a_last_row = 0;   // last valid row of the tile being copied (rows past the end re-read it; they are never stored)
-    auto enter_copy_tile = [&](int j) __attribute__((always_inline)) {
-        const int m0 = (p + j * g.wg_per_group) * C::BM;
-        a_last_row = g.M - 1 - m0;
-        a_tile = uniform_ptr(A + (size_t)m0 * a_row_bytes);
-    };
-    int t_mine = copier ? my_phase : nsteps, t_tile = 0, t_step = my_phase;   // next step this wave copies = step t_step of tile t_tile
-    while (t_step >= ns && ns > 0) {
-        t_step -= ns;
-        ++t_tile;
-    }
-    const unsigned landed_lds = (unsigned)(uintptr_t)(s_landed + (cidx & (NC - 1)));
+    // ---------------- copy side: a wave that waits, copies ----------------
+    // s_next = the first step nobody has copied yet.  A wave that has to wait for a panel (or has no items left) reads all
+    // progress words; while the ring slot of step s_next is free (every wave needs a later step than s_next - RS) it claims
+    // that step with a compare-and-swap on s_next and copies it: 128 rows, then the step's number behind them.  The waves
+    // with few items run ahead, meet steps that are not there yet and so do most of the copying; the waves with many items
+    // only copy when everything has run dry.
+    int* const s_next = s_fail + 1;
+    // t / ns = (t * magic) >> 32 for the step numbers of a workgroup (below 2^16) and 2 <= ns <= 512
+    const unsigned magic_ns = ns > 1 ? 0xFFFFFFFFu / (unsigned)ns + 1u : 0u;
     bool gave_up = false;
     int md = 0;            // last minimum of done[] seen (it only grows)
 
-    auto copy_step = [&]() __attribute__((always_inline)) {   // this wave's rows of step t_mine, then the number t_mine + 1 behind them
-        const int pair = __builtin_amdgcn_readfirstlane(s_steps[t_step]);
-        const unsigned char* src = uniform_ptr(a_tile + (size_t)pair * C::ROWB);
-        const unsigned stage = lds_a + ((unsigned)t_mine % (unsigned)RS) * C::PANEL_BYTES + (unsigned)my_rows * C::ROWB;
-        // (per-lane values are derived again from the lane id behind an opaque copy: kept across the item loop they
+    // Lane l of DMA instruction i of a step: row 8 i + l / 8, physical chunk l % 8 = logical chunk (l % 8) ^ ((row / 2) % 8):
+    // the swizzle term is (l / 16) for even i and (l / 16) ^ 4 for odd i, so two per-lane offsets serve all rows (the row
+    // advances in the scalar base address).
+    auto copy_step = [&](int t) __attribute__((always_inline)) {   // all rows of step t, then the number t + 1 behind them
+        t = __builtin_amdgcn_readfirstlane(t);   // the same in every lane; the DMA helpers want their bases in scalar registers
+        // (tile, step and k-pair are in range by construction; they are clamped all the same, because they make addresses)
+        int tile_c = ns > 1 ? (int)__builtin_amdgcn_readfirstlane((int)__umulhi((unsigned)t, magic_ns)) : t;
+        tile_c = tile_c < ntiles ? tile_c : ntiles - 1;
+        int step_c = t - tile_c * ns;
+        step_c = step_c < 0 ? 0 : (step_c >= ns ? ns - 1 : step_c);
+        const int m0 = (p + tile_c * g.wg_per_group) * C::BM;
+        const int a_last_row = g.M - 1 - m0;   // last valid row of the tile (rows past the end re-read it; they are never stored)
+        int pair = __builtin_amdgcn_readfirstlane(s_steps[step_c]);
+        pair = pair < 0 ? 0 : (pair >= KP ? KP - 1 : pair);
+        const unsigned char* src = uniform_ptr(A + (size_t)m0 * a_row_bytes + (size_t)pair * C::ROWB);
+        const unsigned stage = __builtin_amdgcn_readfirstlane(lds_a + ((unsigned)t % (unsigned)RS) * C::PANEL_BYTES);
+        // (per-lane values are derived from the lane id behind an opaque copy: kept across the item loop they
         // would cost registers the accumulators and fragments need.  A rolled loop: this code must stay small.)
         int lc = lane;
         asm volatile("" : "+v"(lc));
@@ -400,10 +405,10 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
         const unsigned voff_even = voff_row + (unsigned)(((lc & 7) ^ (lc >> 4)) * 16);
         const unsigned voff_odd = voff_row + (unsigned)(((lc & 7) ^ (lc >> 4) ^ 4) * 16);
 #pragma unroll 1
-        for (int i = 0; i < CROWS / 8; i += 2) {
-            const unsigned char* src_i = uniform_ptr(src + (size_t)(my_rows + 8 * i) * a_row_bytes);
-            if (my_rows + 8 * i + 15 <= a_last_row) {
+        for (int i = 0; i < C::BM / 8; i += 2) {
+            if (8 * i + 15 <= a_last_row) {
                 // all 16 rows exist
+                const unsigned char* src_i = uniform_ptr(src + (size_t)(8 * i) * a_row_bytes);
                 dma16(stage + i * 1024, src_i, voff_even);
                 dma16(stage + i * 1024 + 1024, src_i, voff_odd + 8u * a_row_bytes);
             } else {
@@ -411,7 +416,7 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
                 const int l = lc;
 #pragma unroll
                 for (int ii = 0; ii < 2; ++ii) {
-                    const int row = my_rows + 8 * (i + ii) + (l >> 3);
+                    const int row = 8 * (i + ii) + (l >> 3);
                     const int r = row < a_last_row ? row : a_last_row;   // row of the tile, never negative
                     const unsigned voff = (unsigned)r * a_row_bytes + (unsigned)(((l & 7) ^ ((row >> 1) & 7)) * 16);
                     dma16(stage + (i + ii) * 1024, src, voff);
@@ -421,48 +426,26 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
 #ifdef PBS_DDSC_PUBLISH_AFTER_WAIT
         // checking build: wait for the rows, then write the number (relies on no ordering of one wave's loads)
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if (lane == 0) lds_poke(s_landed + cidx, t_mine + 1);
+        if (lane == 0) lds_poke(s_landed + (t & (RS - 1)), t + 1);
 #else
-        dma4_lane0(landed_lds, uniform_ptr(reinterpret_cast<const unsigned char*>(g.seq + (t_mine + 1))));
+        dma4_lane0((unsigned)(uintptr_t)(s_landed + (t & (RS - 1))),
+                   uniform_ptr(reinterpret_cast<const unsigned char*>(g.seq + ((t + 1) & (DC_SEQ_INTS - 1)))));
 #endif
-        t_mine += G;
-        t_step += G;
-        if (t_step >= ns) {
-            do {
-                t_step -= ns;
-                ++t_tile;
-            } while (t_step >= ns);
-            if (t_tile < ntiles) enter_copy_tile(t_tile);
-        }
-    };
-    // Copy this wave's steps whose ring slot is free according to the last done[] minimum seen; never waits.
-    auto try_copy = [&]() __attribute__((always_inline)) {
-        while (t_mine < nsteps && t_mine - RS < md) copy_step();
     };
 
     // ---------------- progress words ----------------
-    // One read: the landed word(s) of the NCS copiers of step u; a copier's lanes 0..15 read done[lane] instead.
-    auto poll_issue = [&](int u) __attribute__((always_inline)) -> int {
-        int off = (u & (G - 1)) * NCS * 4;   // bytes from s_landed
-        if (NCS > 1 || copier) {
-            int l = lane;
-            asm volatile("" : "+v"(l));
-            if (NCS > 1) off += (l & (NCS - 1)) * 4;
-            if (copier) off = l < 16 ? l * 256 - NW * 256 : off;   // done[l] lies NW * 256 bytes before s_landed
-        }
+    // The landed word of step u's ring slot (every lane reads the same word).
+    auto poll_issue = [&](int u) __attribute__((always_inline)) -> int { return lds_peek(s_landed + (u & (RS - 1))); };
+    auto poll_landed = [&](int v, int u) __attribute__((always_inline)) -> bool { return __builtin_amdgcn_readfirstlane(v) > u; };
+    // All progress words in one read: lanes 0..15 done[lane], lane 16 the landed word of step u's slot, lane 17 s_next.
+    auto poll_all = [&](int u) __attribute__((always_inline)) -> int {
+        int l = lane;
+        asm volatile("" : "+v"(l));
+        // byte offsets from s_landed: done[l] lies NW * 256 bytes before it, s_next NC + 1 words behind it
+        const int off = l < 16 ? l * 256 - NW * 256 : (l == 16 ? (u & (RS - 1)) * 4 : (NC + 1) * 4);
         return lds_peek(reinterpret_cast<const int*>(reinterpret_cast<const unsigned char*>(s_landed) + off));
     };
-    // whether step u has landed: all of its copiers count at least u + 1 steps
-    auto poll_landed = [&](int v, int u) __attribute__((always_inline)) -> bool {
-        int m = __builtin_amdgcn_readlane(v, 16);
-#pragma unroll
-        for (int i = 1; i < NCS; ++i) {
-            const int w = __builtin_amdgcn_readlane(v, 16 + i);
-            m = w < m ? w : m;
-        }
-        return m > u;
-    };
-    // a copier also takes the minimum of done[] (-> md)
+    // the minimum of done[] (-> md)
     auto poll_done = [&](int v) __attribute__((always_inline)) {
 #define PBS_MIN_SHR(SH)                                                                \
     {                                                                                  \
@@ -479,17 +462,34 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
         asm volatile("" : "+v"(l));
         lds_poke(s_done + wave * 64 + l, u);
     };
-    // wait until step u has landed, copying what becomes free meanwhile
+    // Copy every step whose ring slot is free and that this wave manages to claim; v = the words poll_all has read.
+    // Returns the value of s_next as far as this wave knows.
+    auto copy_free_steps = [&](int v) __attribute__((always_inline)) -> int {
+        int nc = __builtin_amdgcn_readlane(v, 17);
+        poll_done(v);
+        while (nc < nsteps && nc - RS < md) {
+            int expected = nc;
+            if (lane == 0)
+                __hip_atomic_compare_exchange_strong((lds_int*)s_next, &expected, nc + 1, __ATOMIC_RELAXED,
+                                                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            expected = __builtin_amdgcn_readfirstlane(expected);   // what s_next held: nc if the claim is this wave's
+            if (expected == nc) {
+                copy_step(nc);
+                ++nc;
+            } else {
+                nc = expected;
+            }
+        }
+        return nc;
+    };
+    // wait until step u has landed, copying what is free meanwhile
     auto slow_wait = [&](int u) __attribute__((always_inline)) {
         bool here = false;
         for (int spin = 0; spin < C::SPIN_LIMIT; ++spin) {
-            const int v = poll_issue(u);
-            here = poll_landed(v, u);
-            if (copier) {
-                poll_done(v);
-                try_copy();
-            }
+            const int v = poll_all(u);
+            here = __builtin_amdgcn_readlane(v, 16) > u;
             if (here) break;
+            copy_free_steps(v);
             // another wave has given up: so does this one
             if ((spin & 1023) == 1023 && __builtin_amdgcn_readfirstlane(lds_peek(s_fail)) != 0) break;
             __builtin_amdgcn_s_sleep(DC_SLEEP);
@@ -500,12 +500,11 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
             count_protocol_failure();
         }
     };
-    // after the last item: copy this wave's remaining steps
+    // after the last item: help until every step of the workgroup has been copied
     auto copy_rest = [&]() __attribute__((always_inline)) {
-        for (int spin = 0; spin < C::SPIN_LIMIT && t_mine < nsteps && !gave_up; ++spin) {
+        for (int spin = 0; spin < C::SPIN_LIMIT && !gave_up; ++spin) {
             const int before = md;
-            poll_done(poll_issue(0));
-            try_copy();
+            if (copy_free_steps(poll_all(0)) >= nsteps) break;
             if (md != before) spin = 0;
             if ((spin & 1023) == 1023 && __builtin_amdgcn_readfirstlane(lds_peek(s_fail)) != 0) break;
             __builtin_amdgcn_s_sleep(DC_SLEEP);
@@ -575,9 +574,8 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
         }
     };
 
-    if (copier && ns > 0 && t_tile < ntiles) enter_copy_tile(t_tile);
     if (ns == 0 || ni == 0) {
-        // nothing to multiply in this column: the wave only copies its share of the steps; its result columns are the bias
+        // nothing to multiply in this column: the wave only helps copying; its result columns are the bias
         publish_done(0x7fffffff);
         for (int j = 0; j < ntiles; ++j) epilogue(j);
         if (ns > 0) copy_rest();
@@ -618,15 +616,13 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
     int raw = poll_issue(u);   // the progress words for the item a wave is about to start are read during the previous one
 
 
-    // one item; S = the register set its block was loaded into; COPIER = this wave copies; SMALL = the list is in registers
-    auto do_item = [&](auto S_, auto COPIER_, auto SMALL_) __attribute__((always_inline)) {
+    // one item; S = the register set its block was loaded into; SMALL = the list is in registers
+    auto do_item = [&](auto S_, auto SMALL_) __attribute__((always_inline)) {
         constexpr int S = decltype(S_)::value;
-        constexpr bool COPIER = decltype(COPIER_)::value;
         constexpr bool SMALL = decltype(SMALL_)::value;
         constexpr int SF = (S + L) % (L + 1);
         // has this item's step landed?  (the read is always consumed: one left pending on one path costs a full wait at the join)
         const bool here = poll_landed(raw, u);
-        if constexpr (COPIER) poll_done(raw);
         if (!here && !gave_up) slow_wait(u);   // after a failed wait nothing is waited for any more: the results are void
         // the block of item idx + L, and the next item (behind the last item of the last tile: the list's first again)
         const bool last = (item & DC_ITEM_LAST) != 0;
@@ -655,8 +651,6 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
         for (int t = 0; t < 4; ++t) a0[t] = *reinterpret_cast<const uint4*>(pa0 + t * 4096);
         // the progress words for the next item, behind the fragment reads
         raw = poll_issue(u_n);
-        // (the copy instructions are issued here, right before the wait for this item's block, where they are the youngest)
-        if constexpr (COPIER) try_copy();
         const bf16x8 w0 = __builtin_bit_cast(bf16x8, fb[S][0]);
         const bf16x8 w1 = __builtin_bit_cast(bf16x8, fb[S][1]);
 #pragma unroll
@@ -683,24 +677,19 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
         u_base = u_base_n;
         u = u_n;
     };
-    auto run = [&](auto COPIER_, auto SMALL_) __attribute__((always_inline)) {
+    auto run = [&](auto SMALL_) __attribute__((always_inline)) {
         while (true) {
-            do_item(std::integral_constant<int, 0>{}, COPIER_, SMALL_);
+            do_item(std::integral_constant<int, 0>{}, SMALL_);
             if (j == ntiles) break;
-            do_item(std::integral_constant<int, 1>{}, COPIER_, SMALL_);
+            do_item(std::integral_constant<int, 1>{}, SMALL_);
             if (j == ntiles) break;
-            do_item(std::integral_constant<int, 2>{}, COPIER_, SMALL_);
+            do_item(std::integral_constant<int, 2>{}, SMALL_);
             if (j == ntiles) break;
         }
     };
     static_assert(L == 2, "the item loop is unrolled by L + 1 = 3");
-    if (copier) {
-        if (small) run(std::true_type{}, std::true_type{});
-        else run(std::true_type{}, std::false_type{});
-    } else {
-        if (small) run(std::false_type{}, std::true_type{});
-        else run(std::false_type{}, std::false_type{});
-    }
+    if (small) run(std::true_type{});
+    else run(std::false_type{});
     publish_done(0x7fffffff);
     copy_rest();
 }

@@ -111,7 +111,7 @@ static inline size_t column_plan_bytes(int n, int k) {
 static inline size_t all_plan_bytes(int n, int k) { return column_plan_offset(n, k) + column_plan_bytes(n, k); }
 
 constexpr int D16_TM = 2, D16_RS = 3, D16_RB = 32, D16_NP = 4;
-constexpr double DDSC_MIN_BLOCKS_PER_COLUMN = 40.0;
+constexpr double DDSC_MIN_BLOCKS_PER_COLUMN = 32.0;
 
 // Whether the wide kernel serves this problem: k-pairs need k % 64 == 0, the plan records of a group
 // must fit in LDS beside the rings, and there must be enough tiles to give every CU one.
@@ -157,7 +157,7 @@ static int launch_dds16(const DdsArgs& g, hipStream_t stream) {
 }
 
 // ---- bf16 kernel with one block column per wave ----
-constexpr int DDSC_RS = 8, DDSC_NCS = 1;
+constexpr int DDSC_RS = 8;
 
 // PBS_COLUMN_KERNEL = 0: never use it; 1: whenever it can run; unset: where it is the faster one.
 static int column_kernel_wish() {
@@ -181,8 +181,9 @@ static inline ColumnLaunch column_launch(long long M, int n) {
 }
 
 // Whether that kernel can run this problem at all, and whether it should.  It reads a block's fragments straight
-// from global memory, once per token tile, and pays per step (one k-pair of one tile) what the wide kernel pays,
-// so it wins where the steps are long: many blocks per column.
+// from global memory, once per token tile, and its cost per block product is a third of the wide kernel's while
+// its cost per step (one k-pair of one tile) is about the same: 9 % faster at 32 blocks per column (the
+// 4096 x 4096 layer at density 0.25), 33 % at 64; below that the wide kernel keeps the problem.
 static bool column_kernel_fits(long long M, int n, int k, int nnz, const void* bias) {
     if (!column_plan_bytes(n, k) || nnz < 1 || nnz > DC_MAX_BLOCKS || M < 1) return false;
     if (reinterpret_cast<uintptr_t>(bias) & 3u) return false;
@@ -198,7 +199,7 @@ static bool column_kernel_fits(long long M, int n, int k, int nnz, const void* b
 static int launch_ddsc(const DdsArgs& g, const void* data_nk, hipStream_t stream) {
     using C = DdscCfg<DDSC_RS>;
     static std::atomic<uint64_t> done{0};
-    auto kernel = ddsc_kernel<DDSC_RS, DDSC_NCS>;
+    auto kernel = ddsc_kernel<DDSC_RS>;
     const ColumnLaunch c = column_launch(g.M, g.N);
     DdscArgs a;
     a.a = g.a;

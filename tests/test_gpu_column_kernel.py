@@ -65,6 +65,8 @@ def _check_both_directions(m, tokens, device, seed, what, bias=False):
     (4096, 128, 200, 1.0, False),        # lists of 128 items: more than the two item registers hold
     (1024, 544, 2048 + 1, 0.05, False),  # sparse: columns with no block, steps most columns skip
     (448, 2080, 777, 0.4, True),         # k / 64 = 7 steps, a last group with one column
+    (64, 2048, 128 * 64 * 3 + 50, 0.6, False),   # one step per tile and four tiles per workgroup (steps are numbered across tiles)
+    (192, 4096, 128 * 32 * 2 + 1, 0.3, True),    # three steps per tile, three tiles per workgroup, the last one a single token
 ])
 def test_shapes_against_oracle(cuda, column_kernel, in_f, out_f, tokens, density, bias):
     n_blocks = max(1, int(density * (in_f // 32) * (out_f // 32)))
