@@ -542,14 +542,24 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
         const bool failed = gave_up || __builtin_amdgcn_readfirstlane(lds_peek(s_fail)) != 0;
         int l = lane;
         asm volatile("" : "+v"(l));
-        const int er = l & 31, eh = l >> 5;
+        const int r16 = l & 15, upper = (l >> 4) & 1, eh = l >> 5;
+        // after the exchanges below a lane stores, per token slice, piece (upper, eh) = result columns 8 (2 upper + eh) .. + 7
+        // of token r16 and of token 16 + r16: the four lanes of a token write 64 contiguous bytes in one instruction
+        const int n0 = my_col * 32 + 8 * (2 * upper + eh);
+        uint32_t bw[2][4];
 #pragma unroll
         for (int qq = 0; qq < 2; ++qq) {
-            const int n0 = my_col * 32 + 8 * (2 * qq + eh);   // first of this lane's 8 result columns
             const uint4 braw = *reinterpret_cast<const uint4*>(smem + C::BIAS_OFF + wave * 64 + 16 * (2 * qq + eh));
-            const uint32_t bw[4] = {braw.x, braw.y, braw.z, braw.w};
+            bw[qq][0] = braw.x;
+            bw[qq][1] = braw.y;
+            bw[qq][2] = braw.z;
+            bw[qq][3] = braw.w;
+        }
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
+        for (int t = 0; t < 4; ++t) {
+            uint32_t w[2][4];   // piece qq of this lane's token (lane % 32): result columns 8 (2 qq + eh) .. + 7, as bf16 pairs
+#pragma unroll
+            for (int qq = 0; qq < 2; ++qq) {
                 float x[8];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -560,17 +570,28 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
                     x[e] = __uint_as_float(r[0]);       // column 8 q' + e of this lane's quad q'
                     x[4 + e] = __uint_as_float(r[1]);   // column 8 q' + 4 + e
                 }
-                uint32_t w[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    float lo = x[2 * e] + __uint_as_float(bw[e] << 16);
-                    float hi = x[2 * e + 1] + __uint_as_float(bw[e] & 0xffff0000u);
+                    float lo = x[2 * e] + __uint_as_float(bw[qq][e] << 16);
+                    float hi = x[2 * e + 1] + __uint_as_float(bw[qq][e] & 0xffff0000u);
                     if (failed) lo = hi = __builtin_nanf("");
-                    w[e] = (uint32_t)E::from_f32(lo).bits | ((uint32_t)E::from_f32(hi).bits << 16);
+                    w[qq][e] = (uint32_t)E::from_f32(lo).bits | ((uint32_t)E::from_f32(hi).bits << 16);
                 }
-                const int row = m0 + t * 32 + er;
-                if (row < g.M) *reinterpret_cast<uint4*>(out + (size_t)row * g.N + n0) = make_uint4(w[0], w[1], w[2], w[3]);
             }
+            // The lanes 16..31 of each half hand their piece 0 to the lanes 0..15 and take those lanes' piece 1
+            // (v_permlane16_swap: rows of 16 lanes; the odd rows of the first operand change places with the even rows of
+            // the second).  Then every lane holds one piece of token r16 (first operand) and one of token 16 + r16 (second).
+            uint32_t lo16[4], hi16[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const auto r = __builtin_amdgcn_permlane16_swap(w[0][e], w[1][e], false, false);
+                lo16[e] = r[0];
+                hi16[e] = r[1];
+            }
+            const int row = m0 + t * 32 + r16;
+            if (row < g.M) *reinterpret_cast<uint4*>(out + (size_t)row * g.N + n0) = make_uint4(lo16[0], lo16[1], lo16[2], lo16[3]);
+            if (row + 16 < g.M)
+                *reinterpret_cast<uint4*>(out + (size_t)(row + 16) * g.N + n0) = make_uint4(hi16[0], hi16[1], hi16[2], hi16[3]);
         }
     };
 
