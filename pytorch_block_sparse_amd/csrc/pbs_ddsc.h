@@ -27,7 +27,8 @@
 //                   registers, DC_L items ahead, with ordinary loads (the compiler places the waits and never
 //                   moves a register a load in flight is going to write).  That needs the block stored with
 //                   k along its rows ([n][k]); the stored layout is that for the input gradient, the forward
-//                   product is given a copy of the data with every block transposed (transpose_blocks_kernel).
+//                   product is given a copy of the data with every block transposed (transpose_blocks_kernel),
+//                   which, being a copy anyway, is written in the order the fragments are loaded in.
 //   The LDS so freed makes the panel ring 8 steps deep.
 //
 // The product is computed transposed, acc[n][token] (block fragment as first operand): a lane then holds
@@ -232,7 +233,9 @@ __global__ __launch_bounds__(64) void ddsc_plan_ahead_kernel(int KB, int* plan, 
     }
 }
 
-// data_t block b = data block b transposed (32 x 32 elements of 2 bytes): one wave per block.
+// data_t block b = data block b (stored [k][n], 32 x 32 elements of 2 bytes) in the order ddsc_kernel<RS, true> loads it:
+// [half q of k][lane = 32 h + n][8 k values], k = 16 q + 8 h + e, so that a wave's load of one fragment is 1 KB of
+// consecutive bytes (8 whole cache lines instead of half of each of the block's 16).  One wave per block.
 __global__ __launch_bounds__(256) void transpose_blocks_kernel(const uint16_t* __restrict__ data, uint16_t* __restrict__ data_t,
                                                                int nnz) {
     __shared__ uint16_t s[4][32][34];
@@ -256,15 +259,17 @@ __global__ __launch_bounds__(256) void transpose_blocks_kernel(const uint16_t* _
     uint32_t o[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) o[i] = (uint32_t)s[w][r][c0 + 2 * i] | ((uint32_t)s[w][r][c0 + 2 * i + 1] << 16);
-    *reinterpret_cast<uint4*>(dst + r * 32 + c0) = make_uint4(o[0], o[1], o[2], o[3]);
-    *reinterpret_cast<uint4*>(dst + r * 32 + c0 + 8) = make_uint4(o[4], o[5], o[6], o[7]);
+    // this lane holds k = 16 q .. 16 q + 15 of result column n = r, with q = lane % 2
+    const int q = lane & 1;
+    *reinterpret_cast<uint4*>(dst + q * 512 + r * 8) = make_uint4(o[0], o[1], o[2], o[3]);          // h = 0
+    *reinterpret_cast<uint4*>(dst + q * 512 + (32 + r) * 8) = make_uint4(o[4], o[5], o[6], o[7]);   // h = 1
 }
 
 
 
 struct DdscArgs {
     const void* a;         // [M, K] row-major bf16
-    const void* data;      // [nnz*32, 32] bf16, every block stored [n][k]
+    const void* data;      // [nnz*32, 32] bf16, every block stored [n][k] (FM = false) or in fragment order (FM = true)
     const int* plan;       // built by ddsc_plan_kernel + ddsc_plan_ahead_kernel for this pattern and direction
     const int* seq;        // the table 0, 1, 2, ... written by ddsc_plan_kernel
     const void* bias;      // nullptr or [N]
@@ -301,7 +306,7 @@ static __device__ __forceinline__ void dma4_lane0(unsigned lds_base_uniform, con
                  : "memory");
 }
 
-template <int RS>
+template <int RS, bool FM>
 __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
     static_assert(RS <= DC_NC, "one landed word per ring slot");
     using C = DdscCfg<RS>;
@@ -520,7 +525,8 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
     const unsigned a_pre = (unsigned)(lrow * C::ROWB + ((h ^ ((lrow >> 1) & 7)) * 16));   // offset within a_ring
     static_assert((RS & (RS - 1)) == 0, "the ring slot is a bit field of the address");
     // block fragment q: row lrow of the [n][k] block, 16 bytes at 16 (2 q + h)
-    const unsigned b_lane = (unsigned)(lrow * 64 + h * 16);
+    // (or, in fragment order, 16 bytes at 1024 q + 16 lane)
+    const unsigned b_lane = FM ? (unsigned)(lane * 16) : (unsigned)(lrow * 64 + h * 16);
 
     bf16_t* out = static_cast<bf16_t*>(g.out);
 
@@ -610,7 +616,7 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
         // plain loads: the compiler places the wait before their first use
         const unsigned char* pb = Dp + (size_t)(byte_off + b_lane);
         b0 = *reinterpret_cast<const u32x4*>(pb);
-        b1 = *reinterpret_cast<const u32x4*>(pb + 32);
+        b1 = *reinterpret_cast<const u32x4*>(pb + (FM ? 1024 : 32));
     };
     // the blocks of the first L items: item i's block offset is the second word of item i - L (cyclically)
 #pragma unroll

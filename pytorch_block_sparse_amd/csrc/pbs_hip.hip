@@ -196,10 +196,12 @@ static bool column_kernel_fits(long long M, int n, int k, int nnz, const void* b
     return (double)nnz / (n / 32) >= DDSC_MIN_BLOCKS_PER_COLUMN;
 }
 
+// FM: the blocks are given in fragment order (the forward product's copy) instead of [n][k] as stored
+template <bool FM>
 static int launch_ddsc(const DdsArgs& g, const void* data_nk, hipStream_t stream) {
     using C = DdscCfg<DDSC_RS>;
     static std::atomic<uint64_t> done{0};
-    auto kernel = ddsc_kernel<DDSC_RS>;
+    auto kernel = ddsc_kernel<DDSC_RS, FM>;
     const ColumnLaunch c = column_launch(g.M, g.N);
     DdscArgs a;
     a.a = g.a;
@@ -236,13 +238,13 @@ static int dispatch_dds(const DdsArgs& g, void* workspace, size_t workspace_byte
     if constexpr (sizeof(T) == 2) {
         if (column_kernel_fits(g.M, g.N, g.K, g.nnz, g.bias)) {
             // the kernel wants every block with k along its rows: as stored for TRANS, a transposed copy otherwise
-            if constexpr (TRANS) return launch_ddsc(g, g.data, stream);
+            if constexpr (TRANS) return launch_ddsc<false>(g, g.data, stream);
             const size_t need = (size_t)g.nnz * 2048;
             if (workspace && workspace_bytes >= need && aligned16(workspace)) {
                 hipLaunchKernelGGL(transpose_blocks_kernel, dim3((unsigned)((g.nnz + 3) / 4)), dim3(256), 0, stream,
                                    static_cast<const uint16_t*>(g.data), static_cast<uint16_t*>(workspace), g.nnz);
                 if (int rc = (int)hipGetLastError()) return rc;
-                return launch_ddsc(g, workspace, stream);
+                return launch_ddsc<true>(g, workspace, stream);
             }
         }
         if (wide_kernel_fits(g.M, g.N, g.K)) return launch_dds16<TRANS>(g, stream);
