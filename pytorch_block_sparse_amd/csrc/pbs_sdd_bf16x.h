@@ -230,6 +230,7 @@ __global__ __launch_bounds__(512) void sdd_bf16x_kernel(SddArgs a) {
         // copies waits for its loads before it goes on) and every wave has left the last chunk's buffer
         __syncthreads();
         if (tid < NW + NS + 2) s_done[tid] = 0;
+        md = 0;
         __syncthreads();
 
         auto load_frag = [&](uint4& f, const unsigned char* p) __attribute__((always_inline)) {
