@@ -15,7 +15,6 @@
 #include "pbs_index.h"
 #include "pbs_sdd.h"
 #include "pbs_sdd_bf16.h"
-#include "pbs_sdd_bf16x.h"
 #include "pbs_sdd_seg.h"
 
 namespace pbs {
@@ -459,13 +458,6 @@ static int launch_sdd_seg(const SddArgs& a, long long wgs, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
-// PBS_DW_KERNEL = 1: the bf16 weight gradient without barriers in the token loop (pbs_sdd_bf16x.h); otherwise the
-// kernel with a barrier per chunk (pbs_sdd_bf16.h).
-static bool barrier_free_dw() {
-    const char* e = std::getenv("PBS_DW_KERNEL");
-    return e && e[0] == '1';
-}
-
 template <typename T>
 static int launch_sdd(SddArgs a, int dtype, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     const SddPlan p = plan_sdd_for(dtype, a.M, a.N, a.K, a.nnz);
@@ -490,22 +482,12 @@ static int launch_sdd(SddArgs a, int dtype, void* workspace, size_t workspace_by
         if (rc) return rc;
     } else {
         using S = SddShapeBf16;
-        if (barrier_free_dw()) {
-            // no barriers in the token loop; chunks of 16 tokens (the plan's slices are multiples of 32 tokens)
-            using C = SddBf16xCfg<S::QW>;
-            static_assert(S::TC % C::TC == 0 && C::SR == S::SR && C::SC == S::SC, "plan and kernel must agree");
-            static std::atomic<uint64_t> done{0};
-            auto kernel = sdd_bf16x_kernel<S::QW>;
-            if (int rc = raise_lds_limit(kernel, C::LDS_BYTES, done)) return rc;
-            hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)wgs)), dim3(C::NT), C::LDS_BYTES, stream, a);
-        } else {
-            using C = SddBf16Cfg<S::QW, S::TC, S::NS, S::NW>;
-            static_assert(C::TC == S::TC && C::SR == S::SR && C::SC == S::SC, "plan and kernel must agree");
-            static std::atomic<uint64_t> done{0};
-            auto kernel = sdd_bf16_kernel<S::QW, S::TC, S::NS, S::NW>;
-            if (int rc = raise_lds_limit(kernel, C::LDS_BYTES, done)) return rc;
-            hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)wgs)), dim3(C::NT), C::LDS_BYTES, stream, a);
-        }
+        using C = SddBf16Cfg<S::QW, S::TC, S::NS, S::NW>;
+        static_assert(C::TC == S::TC && C::SR == S::SR && C::SC == S::SC, "plan and kernel must agree");
+        static std::atomic<uint64_t> done{0};
+        auto kernel = sdd_bf16_kernel<S::QW, S::TC, S::NS, S::NW>;
+        if (int rc = raise_lds_limit(kernel, C::LDS_BYTES, done)) return rc;
+        hipLaunchKernelGGL(kernel, dim3(xcd_grid((int)wgs)), dim3(C::NT), C::LDS_BYTES, stream, a);
     }
     int rc = (int)hipGetLastError();
     if (rc) return rc;
