@@ -271,11 +271,11 @@ __global__ __launch_bounds__(NW * 64) void sdd_seg_kernel(SddArgs a) {
         for (int q0 = 0; q0 < nq; q0 += C::QMAX) {
             // this pass: blocks [q0, q0 + npass), dealt to the waves in contiguous runs
             const int npass = (nq - q0 < C::QMAX) ? nq - q0 : C::QMAX;
-            const int per = (npass + NW - 1) / NW;
-            const int w_lo = q0 + wave * per;
-            int w_n = q0 + npass - w_lo;
-            if (w_n > per) w_n = per;
-            if (w_n < 0) w_n = 0;
+            // (runs of npass / NW blocks, the first npass % NW waves one more: waves w and w + 4 share a SIMD, so the
+            // longer runs spread over the SIMDs)
+            const int per = npass / NW, rem = npass % NW;
+            const int w_lo = q0 + wave * per + (wave < rem ? wave : rem);
+            const int w_n = per + (wave < rem ? 1 : 0);
 
             f32x16 acc[QW];
 #pragma unroll
