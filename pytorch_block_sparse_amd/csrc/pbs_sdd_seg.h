@@ -303,8 +303,9 @@ __global__ __launch_bounds__(NW * 64) void sdd_seg_kernel(SddArgs a) {
                     bv[s] = __uint_as_float(pb[s * FG]);
                 }
             };
-            // next_ci >= 0: this wave's share of the DMA of that chunk is issued behind the first block's products,
-            // so that the matrix cores are already busy while the wave spends its issue slots on the DMA
+            // next_ci >= 0: this wave's share of the DMA of that chunk is issued behind the first (upper four waves:
+            // second) block's products, so that the matrix cores are already busy while the wave spends its issue
+            // slots on the DMA
             auto compute_chunk = [&](int buf, int next_ci) __attribute__((always_inline)) {
                 const uint32_t* sg = reinterpret_cast<const uint32_t*>(stage0 + buf * C::STAGE_BYTES);
                 const uint32_t* sx = reinterpret_cast<const uint32_t*>(stage0 + buf * C::STAGE_BYTES + C::G_BYTES);
@@ -320,10 +321,13 @@ __global__ __launch_bounds__(NW * 64) void sdd_seg_kernel(SddArgs a) {
             _Pragma("unroll") for (int s = 0; s < 8; ++s)                                                             \
                 acc[(I) % QW] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[(I) & 1][s], bv[(I) & 1][s], acc[(I) % QW], 0, 0, 0); \
             __builtin_amdgcn_sched_barrier(0);                                                                        \
-            if ((I) == 0 && next_ci >= 0) dma_chunk(next_ci, next_ci & 1);
+            if ((I) < 2 && (I) == dma_at && next_ci >= 0) dma_chunk(next_ci, next_ci & 1);
 #define PBS_SEG_END }}
 
                 static_assert(QW <= 10, "the nest below has ten levels");
+                // the two waves of a SIMD copy at different times (the upper four waves one block later): while one is
+                // held by the texture path the other has products to issue
+                const int dma_at = (wave >= NW / 2 && w_n > 1) ? 1 : 0;
                 if (w_n > 0) {
                     fetch_frags(sg, sx, pos[0], av[0], bv[0]);
                     PBS_SEG_BLOCK(0) PBS_SEG_BLOCK(1) PBS_SEG_BLOCK(2) PBS_SEG_BLOCK(3) PBS_SEG_BLOCK(4)
