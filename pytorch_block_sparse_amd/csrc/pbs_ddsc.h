@@ -605,9 +605,17 @@ __global__ __launch_bounds__(DC_NB * 64) void ddsc_kernel(DdscArgs g) {
                 hi16[e] = r[1];
             }
             const int row = m0 + t * 32 + r16;
-            if (row < g.M) *reinterpret_cast<uint4*>(out + (size_t)row * g.N + n0) = make_uint4(lo16[0], lo16[1], lo16[2], lo16[3]);
-            if (row + 16 < g.M)
-                *reinterpret_cast<uint4*>(out + (size_t)(row + 16) * g.N + n0) = make_uint4(hi16[0], hi16[1], hi16[2], hi16[3]);
+            // Non-temporal stores: the result (128 MiB at the benchmark shape) is not read again by this kernel, and
+            // written the ordinary way it pushes the operands of the next product out of the last-level cache (the
+            // weight gradient behind the input gradient 0.223 -> 0.207 ms, the whole step 0.589 -> 0.566).
+            if (row < g.M) {
+                const u32x4 vlo = {lo16[0], lo16[1], lo16[2], lo16[3]};
+                __builtin_nontemporal_store(vlo, reinterpret_cast<u32x4*>(out + (size_t)row * g.N + n0));
+            }
+            if (row + 16 < g.M) {
+                const u32x4 vhi = {hi16[0], hi16[1], hi16[2], hi16[3]};
+                __builtin_nontemporal_store(vhi, reinterpret_cast<u32x4*>(out + (size_t)(row + 16) * g.N + n0));
+            }
         }
     };
 
