@@ -378,11 +378,10 @@ __global__ __launch_bounds__(256) void sdd_reduce_kernel(const float* partial, T
     using E = Elem<T>;
     const size_t i4 = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i4 >= n) return;   // n is a multiple of 1024
-    float4 s = *reinterpret_cast<const float4*>(partial + i4);
-    for (int k = 1; k < nsplit; ++k) {
-        const float4 p = *reinterpret_cast<const float4*>(partial + (size_t)k * n + i4);
-        s.x += p.x; s.y += p.y; s.z += p.z; s.w += p.w;
-    }
+    // non-temporal loads: the partial sums are not read again
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    f32x4 s = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(partial + i4));
+    for (int k = 1; k < nsplit; ++k) s += __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(partial + (size_t)k * n + i4));
     out[i4 + 0] = E::from_f32(s.x);
     out[i4 + 1] = E::from_f32(s.y);
     out[i4 + 2] = E::from_f32(s.z);

@@ -473,7 +473,9 @@ __global__ __launch_bounds__(NW_ * 64) void sdd_bf16_kernel(SddArgs a) {
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const size_t o = (size_t)blk_of[q] * 1024 + acc_row(v, h) * 32 + lrow;
-                    if (part) part[o] = acc[q][v];
+                    // (partial sums are written once and read once, by sdd_reduce_kernel: stored and loaded non-temporally
+                    // they leave the operands of the next product in the last-level cache)
+                    if (part) __builtin_nontemporal_store(acc[q][v], part + o);
                     else out[o] = Elem<bf16_t>::from_f32(acc[q][v]);
                 }
             }
