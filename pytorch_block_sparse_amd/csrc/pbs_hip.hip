@@ -112,6 +112,7 @@ static inline size_t all_plan_bytes(int n, int k) { return column_plan_offset(n,
 
 constexpr int D16_TM = 2, D16_RS = 3, D16_RB = 32, D16_NP = 4;
 constexpr double DDSC_MIN_BLOCKS_PER_COLUMN = 32.0;
+constexpr int DDSC_WIDE_RESULT = 2048;
 
 // Whether the wide kernel serves this problem: k-pairs need k % 64 == 0, the plan records of a group
 // must fit in LDS beside the rings, and there must be enough tiles to give every CU one.
@@ -181,9 +182,12 @@ static inline ColumnLaunch column_launch(long long M, int n) {
 }
 
 // Whether that kernel can run this problem at all, and whether it should.  It reads a block's fragments straight
-// from global memory, once per token tile, and its cost per block product is a third of the wide kernel's while
-// its cost per step (one k-pair of one tile) is about the same: 9 % faster at 32 blocks per column (the
-// 4096 x 4096 layer at density 0.25), 33 % at 64; below that the wide kernel keeps the problem.
+// from global memory, once per token tile, and its cost per block product is a third of the wide kernel's: 20 %
+// faster at 32 blocks per column (the 4096 x 4096 layer at density 0.25), 35 % at 64.  Measured over densities
+// 0.008 to 1 and results 512 to 4096 wide (16384 tokens): with a result of 2048 columns or more it is also the
+// faster one for sparse patterns (4096 x 4096: 6 to 30 % at 1 to 24 blocks per column; 2048 x 2048: level at 2 to 4
+// blocks per column, 5 to 13 % from 8), while results of 512 to 1024 columns stay 10 to 30 % faster in the other
+// kernels until their columns hold 32 blocks.
 static bool column_kernel_fits(long long M, int n, int k, int nnz, const void* bias) {
     if (!column_plan_bytes(n, k) || nnz < 1 || nnz > DC_MAX_BLOCKS || M < 1) return false;
     if (reinterpret_cast<uintptr_t>(bias) & 3u) return false;
@@ -193,7 +197,12 @@ static bool column_kernel_fits(long long M, int n, int k, int nnz, const void* b
     const int wish = column_kernel_wish();
     if (wish >= 0) return wish == 1;
     if ((long long)c.m_tiles * c.n_groups < 256) return false;
-    return (double)nnz / (n / 32) >= DDSC_MIN_BLOCKS_PER_COLUMN;
+    const double per_column = (double)nnz / (n / 32);
+    if (per_column >= DDSC_MIN_BLOCKS_PER_COLUMN) return true;
+    // wide results (at least four groups of 16 block columns): from 16 blocks per column, and from 2 when the contraction
+    // is long enough for the ring to fill (16 k-pairs)
+    if (n >= DDSC_WIDE_RESULT && per_column >= 16.0) return true;
+    return n >= DDSC_WIDE_RESULT && k >= 1024 && per_column >= 2.0;
 }
 
 // FM: the blocks are given in fragment order (the forward product's copy) instead of [n][k] as stored

@@ -76,7 +76,11 @@ def test_matmul_workspace_entry_point(lib):
     assert ws(16384, 4096, 4096, 8192, 1, 1) == 8192 * 2048
     assert ws(16384, 4096, 4096, 8192, 0, 1) == 0      # the input gradient reads the data as stored
     assert ws(16384, 4096, 4096, 8192, 1, 0) == 0      # fp32
-    assert ws(16384, 4096, 4096, 400, 1, 1) == 0       # 3 blocks per column
+    assert ws(16384, 4096, 4096, 400, 1, 1) == 400 * 2048   # 3 blocks per column of a result of 4096 columns: still that kernel
+    assert ws(16384, 4096, 4096, 128, 1, 1) == 0       # 1 block per column
+    assert ws(16384, 1024, 4096, 512, 1, 1) == 0       # a result of 1024 columns at 16 blocks per column
+    assert ws(16384, 2048, 512, 640, 1, 1) == 0        # a short contraction below 16 blocks per column
+    assert ws(16384, 2048, 512, 1024, 1, 1) == 1024 * 2048   # ... and at 16
     assert ws(256, 4096, 4096, 8192, 1, 1) == 0        # too few tiles
     assert ws(16384, 4096, 8192, 16384, 1, 1) == 0     # contraction too long for the kernel's lists
     assert ws(16384, 4096, 4096, 0, 1, 1) == 0 and ws(0, 4096, 4096, 8192, 1, 1) == 0

@@ -150,3 +150,19 @@ def test_without_workspace_the_forward_product_still_runs(cuda, column_kernel):
     y_ref = to64(x) @ O.to_dense(to64(m.data), coo, (out_f, in_f)).T
     assert_close(out, y_ref, BF16, "no workspace")
     assert_close(y, y_ref, BF16, "workspace")
+
+
+def test_sparse_wide_layer_takes_the_column_kernel_by_itself(cuda, monkeypatch):
+    """2048 -> 2048 at density 0.06 (4 blocks per column), 8229 tokens: a result of 2048 columns and a contraction of
+    32 k-pairs go to the column kernel without being forced, in both directions; checked against the oracle in full."""
+    monkeypatch.delenv("PBS_COLUMN_KERNEL", raising=False)
+    out_f = in_f = 2048
+    tokens = 8192 + 37
+    m = _matrix(out_f, in_f, None, int(0.06 * 64 * 64), cuda, seed=12)
+    name = native.matmul_kernel_name(tokens, out_f, in_f, m.cols_a.shape[0], True, BF16)
+    assert "ddsc" in name, name
+    name = native.matmul_kernel_name(tokens, in_f, out_f, m.cols_a.shape[0], False, BF16)
+    assert "ddsc" in name, name
+    _check_both_directions(m, tokens, cuda, 5, "sparse wide layer", bias=True)
+    # a result of 1024 columns at the same density stays with the other kernels
+    assert "ddsc" not in native.matmul_kernel_name(16384, 1024, 4096, int(0.06 * 32 * 128), True, BF16)
